@@ -1,0 +1,2 @@
+"""A small, whole inference engine for one GPU of the MI355X kind (gfx950), with hand-written HIP kernels."""
+__version__ = "0.1.0"

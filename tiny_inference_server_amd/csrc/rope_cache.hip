@@ -1,0 +1,76 @@
+// Rotary position encoding of queries and keys, fused with the write of keys and values into cache pages.
+//
+// Input rows hold [q heads | k heads | v heads] as one projection wrote them. Queries are rotated in place,
+// keys are rotated on their way into the page, values are copied. The rotation runs in 32-bit on a table of
+// (cos, sin) per position and pair. Pairs are (j, j + head_dim/2) in the "half" pairing (reference
+// main_models_new.py:71-80) or (2j, 2j+1) in the "interleaved" pairing; a null table means no rotation.
+//
+// One cache plane is laid out [page][key or value][kv head][slot in page][head_dim].
+#include "common.h"
+
+TIS_DEFINE_LAST_ERROR(tis_rope_cache)
+
+template <typename T>
+__global__ __launch_bounds__(64) void rope_write_kv_kernel(T* __restrict__ qkv, long ld, const int* __restrict__ positions,
+                                                           const int* __restrict__ write_slots,
+                                                           const float2* __restrict__ table, T* __restrict__ plane,
+                                                           int n_heads, int n_kv_heads, int head_dim, int page_size,
+                                                           int interleaved, int write_cache) {
+  const long r = blockIdx.x;
+  const int hh = blockIdx.y;  // [0, n_heads): q, then k heads, then v heads
+  const int half = head_dim / 2;
+  T* row = qkv + r * ld + (long)hh * head_dim;
+
+  T* dst = row;  // queries are rewritten where they are
+  const bool is_q = hh < n_heads;
+  const bool is_v = hh >= n_heads + n_kv_heads;
+  if (!is_q) {
+    if (!write_cache) {
+      if (is_v) return;  // nothing to do for values
+    } else {
+      const int slot = write_slots[r];
+      const int page = slot / page_size, off = slot % page_size;
+      const int kvh = is_v ? hh - n_heads - n_kv_heads : hh - n_heads;
+      dst = plane + ((((long)page * 2 + (is_v ? 1 : 0)) * n_kv_heads + kvh) * page_size + off) * head_dim;
+    }
+  }
+  if (is_v || table == nullptr) {
+    if (dst != row)
+      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = row[i];
+    return;
+  }
+  const float2* cs = table + (long)positions[r] * half;
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    const int a = interleaved ? 2 * j : j;
+    const int b = interleaved ? 2 * j + 1 : j + half;
+    const float x1 = to_f(row[a]), x2 = to_f(row[b]);
+    const float c = cs[j].x, s = cs[j].y;
+    // q*cos + rotate_half(q)*sin with rotate_half = [-x2, x1]
+    const float y1 = x1 * c - x2 * s;
+    const float y2 = x2 * c + x1 * s;
+    dst[a] = from_f<T>(y1);
+    dst[b] = from_f<T>(y2);
+  }
+}
+
+TIS_EXPORT int tis_rope_write_kv(int dtype, void* qkv, long ld, const int* positions, const int* write_slots,
+                                 const float* table, void* plane, int rows, int n_heads, int n_kv_heads, int head_dim,
+                                 int page_size, int interleaved, int write_cache, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || n_heads < 1 || n_kv_heads < 1 || head_dim < 2 || (head_dim & 1) || page_size < 1)
+    return tis_fail("rope_write_kv: bad size rows=%d heads=%d kv_heads=%d head_dim=%d page=%d", rows, n_heads,
+                    n_kv_heads, head_dim, page_size);
+  if (n_heads + 2 * n_kv_heads > 65535) return tis_fail("rope_write_kv: too many heads for the grid");
+  dim3 grid(rows, n_heads + 2 * n_kv_heads);
+  if (dtype == TIS_F32)
+    rope_write_kv_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, ld, positions, write_slots, (const float2*)table,
+                                                         (float*)plane, n_heads, n_kv_heads, head_dim, page_size,
+                                                         interleaved, write_cache);
+  else if (dtype == TIS_BF16)
+    rope_write_kv_kernel<bf16><<<grid, 64, 0, stream>>>((bf16*)qkv, ld, positions, write_slots, (const float2*)table,
+                                                        (bf16*)plane, n_heads, n_kv_heads, head_dim, page_size,
+                                                        interleaved, write_cache);
+  else
+    return tis_fail("unknown dtype code %d", dtype);
+  return tis_launch_status("rope_write_kv");
+}

@@ -1,0 +1,218 @@
+// Token sampling, one workgroup per row of logits, all in 32-bit.
+//
+// Order of operations as in the reference's batch_probs (server.py:22-50): repetition penalty on the
+// tokens of the request's context (l > 0 ? l / pen : l * pen, each token once) -> divide by the
+// temperature -> top-k -> top-p (keep a token while the probability mass of the strictly larger ones is
+// <= top_p, so the token that crosses top_p stays) -> softmax over what is left -> draw.
+// The reference sorts; here both cuts are thresholds found by bisection over the bit pattern of the
+// values, which keeps the same set whenever the values at the cut are distinct (ties at the top-k cut
+// are all kept). The draw takes a uniform number per row from the caller (a stream per request, so a
+// request's tokens do not depend on what else is in the batch) and inverts the cumulative distribution
+// in token order. temperature == 0 or top_k == 1 is greedy: the arg-max, lowest index on ties.
+#include "common.h"
+
+TIS_DEFINE_LAST_ERROR(tis_sampling)
+
+static constexpr int SM_THREADS = 1024;
+
+__device__ __forceinline__ unsigned order_key(float v) {
+  unsigned u = __float_as_uint(v);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// (value, index) arg-max over the block; lowest index wins ties. Result valid in every thread.
+__device__ __forceinline__ void block_argmax(float& v, int& ix, float* sv, int* si) {
+#pragma unroll
+  for (int o = TIS_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, TIS_WAVE);
+    const int oi = __shfl_xor(ix, o, TIS_WAVE);
+    if (ov > v || (ov == v && oi < ix)) { v = ov; ix = oi; }
+  }
+  const int wave = threadIdx.x / TIS_WAVE, lane = threadIdx.x % TIS_WAVE;
+  __syncthreads();
+  if (lane == 0) { sv[wave] = v; si[wave] = ix; }
+  __syncthreads();
+  v = sv[0]; ix = si[0];
+  for (int i = 1; i < SM_THREADS / TIS_WAVE; ++i)
+    if (sv[i] > v || (sv[i] == v && si[i] < ix)) { v = sv[i]; ix = si[i]; }
+}
+
+__global__ __launch_bounds__(SM_THREADS) void sample_kernel(
+    const float* __restrict__ logits, long ld, float* __restrict__ work, int V, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ rep_penalty,
+    const int* __restrict__ ctx_tokens, const int* __restrict__ ctx_offsets, const float* __restrict__ uniform,
+    int* __restrict__ out_tokens) {
+  __shared__ float red[16];
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  __shared__ float part[SM_THREADS];
+  __shared__ int found;
+  __shared__ int first_owner;
+
+  const long r = blockIdx.x;
+  const int t = threadIdx.x;
+  const float* lg = logits + r * ld;
+  float* x = work + r * (long)V;
+  const float temp = temperature[r];
+  const int k_req = top_k[r];
+  const float p_req = top_p[r];
+  const float pen = rep_penalty ? rep_penalty[r] : 1.f;
+  const bool greedy = (temp == 0.f) || (k_req == 1);
+  const float inv_t = greedy ? 1.f : 1.f / temp;
+
+  for (int i = t; i < V; i += SM_THREADS) x[i] = lg[i] * inv_t;
+  __syncthreads();
+  if (pen != 1.f && ctx_tokens) {
+    // computed from the untouched logits, so a token that occurs twice is still penalised once
+    for (int c = ctx_offsets[r] + t; c < ctx_offsets[r + 1]; c += SM_THREADS) {
+      const int tok = ctx_tokens[c];
+      if (tok >= 0 && tok < V) {
+        const float l = lg[tok];
+        x[tok] = (l > 0.f ? l / pen : l * pen) * inv_t;
+      }
+    }
+    __syncthreads();
+  }
+
+  // maximum and its index
+  float mv = -INFINITY;
+  int mi = 0x7fffffff;
+  for (int i = t; i < V; i += SM_THREADS) {
+    const float v = x[i];
+    if (v > mv) { mv = v; mi = i; }
+  }
+  block_argmax(mv, mi, sv, si);
+  if (mi < 0 || mi >= V) mi = 0;  // only when every value is NaN
+  if (greedy) {
+    if (t == 0) out_tokens[r] = mi;
+    return;
+  }
+
+  // top-k: the k-th largest key, built bit by bit
+  unsigned cut = 0u;
+  if (k_req > 0 && k_req < V) {
+    for (int bit = 31; bit >= 0; --bit) {
+      const unsigned cand = cut | (1u << bit);
+      float cnt = 0.f;
+      for (int i = t; i < V; i += SM_THREADS) cnt += (order_key(x[i]) >= cand) ? 1.f : 0.f;
+      cnt = block_sum(cnt, red);
+      if (cnt >= (float)k_req) cut = cand;
+    }
+  }
+  float z = 0.f;
+  for (int i = t; i < V; i += SM_THREADS) {
+    const float v = x[i];
+    if (order_key(v) >= cut) z += expf(v - mv);
+  }
+  z = block_sum(z, red);
+
+  // top-p: the largest key whose mass at or above it exceeds top_p
+  if (p_req > 0.f && p_req < 1.f) {
+    unsigned pc = 0u;
+    const float limit = p_req * z;
+    for (int bit = 31; bit >= 0; --bit) {
+      const unsigned cand = pc | (1u << bit);
+      float mass = 0.f;
+      for (int i = t; i < V; i += SM_THREADS) {
+        const float v = x[i];
+        const unsigned key = order_key(v);
+        if (key >= cand && key >= cut) mass += expf(v - mv);
+      }
+      mass = block_sum(mass, red);
+      if (mass > limit) pc = cand;
+    }
+    if (pc > cut) {
+      cut = pc;
+      z = 0.f;
+      for (int i = t; i < V; i += SM_THREADS) {
+        const float v = x[i];
+        if (order_key(v) >= cut) z += expf(v - mv);
+      }
+      z = block_sum(z, red);
+    }
+  }
+
+  // inverse CDF in token order: thread t owns the tokens [t*chunk, (t+1)*chunk)
+  const int chunk = (V + SM_THREADS - 1) / SM_THREADS;
+  const int lo = min(V, t * chunk), hi = min(V, lo + chunk);
+  float mine = 0.f;
+  for (int i = lo; i < hi; ++i) {
+    const float v = x[i];
+    if (order_key(v) >= cut) mine += expf(v - mv);
+  }
+  part[t] = mine;
+  if (t == 0) { found = -1; first_owner = SM_THREADS; }
+  __syncthreads();
+  if (t < TIS_WAVE) {
+    // one wave scans the 1024 partial sums in order: 16 per lane, then across lanes
+    float s = 0.f;
+    for (int i = 0; i < SM_THREADS / TIS_WAVE; ++i) s += part[t * (SM_THREADS / TIS_WAVE) + i];
+    float incl = s;
+#pragma unroll
+    for (int o = 1; o < TIS_WAVE; o <<= 1) {
+      const float up = __shfl_up(incl, o, TIS_WAVE);
+      if (t >= o) incl += up;
+    }
+    float run = incl - s;
+    for (int i = 0; i < SM_THREADS / TIS_WAVE; ++i) {
+      const int ix = t * (SM_THREADS / TIS_WAVE) + i;
+      const float v = part[ix];
+      part[ix] = run;  // exclusive prefix
+      run += v;
+    }
+  }
+  __syncthreads();
+  // the owner of the draw is the first thread whose running total passes the target; taking the minimum
+  // over candidates keeps the choice well defined where rounding makes neighbouring intervals overlap
+  const float target = uniform[r] * z;
+  const float before = part[t];
+  if (mine > 0.f && before + mine > target) atomicMin(&first_owner, t);
+  __syncthreads();
+  if (t == first_owner) {
+    float run = before;
+    int pick = -1;
+    for (int i = lo; i < hi; ++i) {
+      const float v = x[i];
+      if (order_key(v) >= cut) {
+        run += expf(v - mv);
+        pick = i;
+        if (run > target) break;
+      }
+    }
+    found = pick;
+  }
+  __syncthreads();
+  if (t == 0) out_tokens[r] = found >= 0 ? found : mi;  // rounding left the target past the last token: take the mode
+}
+
+TIS_EXPORT int tis_sample(const float* logits, long ld, float* work, int rows, int V, const float* temperature,
+                          const int* top_k, const float* top_p, const float* rep_penalty, const int* ctx_tokens,
+                          const int* ctx_offsets, const float* uniform, int* out_tokens, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || V < 1) return tis_fail("sample: bad size rows=%d vocab=%d", rows, V);
+  sample_kernel<<<rows, SM_THREADS, 0, stream>>>(logits, ld, work, V, temperature, top_k, top_p, rep_penalty,
+                                                 ctx_tokens, ctx_offsets, uniform, out_tokens);
+  return tis_launch_status("sample");
+}
+
+__global__ __launch_bounds__(SM_THREADS) void argmax_kernel(const float* __restrict__ logits, long ld, int V,
+                                                            int* __restrict__ out_tokens) {
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  const long r = blockIdx.x;
+  float mv = -INFINITY;
+  int mi = 0x7fffffff;
+  for (int i = threadIdx.x; i < V; i += SM_THREADS) {
+    const float v = logits[r * ld + i];
+    if (v > mv) { mv = v; mi = i; }
+  }
+  block_argmax(mv, mi, sv, si);
+  if (threadIdx.x == 0) out_tokens[r] = (mi < 0 || mi >= V) ? 0 : mi;
+}
+
+TIS_EXPORT int tis_argmax(const float* logits, long ld, int rows, int V, int* out_tokens, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || V < 1) return tis_fail("argmax: bad size rows=%d vocab=%d", rows, V);
+  argmax_kernel<<<rows, SM_THREADS, 0, stream>>>(logits, ld, V, out_tokens);
+  return tis_launch_status("argmax");
+}

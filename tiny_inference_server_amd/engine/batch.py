@@ -1,0 +1,185 @@
+"""The rows of one step, as the kernels want them.
+
+A step brings, for some live requests, their next tokens: a request that was fed positions [0, s) and
+now brings n tokens contributes the rows of positions [s, s+n). A stage of lag j (stage 0 is the trunk)
+runs, for the same entry, the positions [max(0, s-j), s+n-j): the same tokens, shifted. Every stage gets
+its own row arrays; the block tables are the same for all stages because they describe the requests, not
+the rows. All integer arrays of a step are packed into one host buffer and copied to the device once.
+
+Per stage:
+  tokens[r], positions[r]      the row's token and absolute position
+  row_seq[r]                   index of the row's entry (its line in the block tables)
+  cu_rows[k], cu_rows[k+1]     the rows of entry k
+  write_slots[group][r]        page * page_size + offset where the row's key and value go
+  source_index[r]              for stages that read the previous stage: its row index there, or -(slot+1)
+                               for the row kept in the request's state slot
+  keep_source[i], keep_slot[i] previous-stage rows to keep in state slots after the reads
+  want_index[i]                the rows whose outputs are asked for (-1 where this stage has no such row yet)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+
+@dataclass
+class Entry:
+    slot: int                  # request slot in the cache manager
+    start: int                 # position of the first token
+    tokens: Sequence[int]
+    want: Sequence[int] = ()   # indices into `tokens`
+
+
+@dataclass
+class StageBatch:
+    lag: int
+    n_rows: int
+    n_seqs: int
+    tokens: torch.Tensor
+    positions: torch.Tensor
+    row_seq: torch.Tensor
+    cu_rows: torch.Tensor
+    seq_slots: torch.Tensor
+    write_slots: Dict[str, torch.Tensor]
+    block_tables: Dict[str, torch.Tensor]
+    source_index: Optional[torch.Tensor]
+    keep_source: Optional[torch.Tensor]
+    keep_slot: Optional[torch.Tensor]
+    keep_count: int
+    want_index: torch.Tensor
+    want_valid: List[bool]
+    max_kv_len: int
+    max_seq_rows: int
+    seq_rows: List[Tuple[int, int, int]]      # host copy: (first row, first position, rows) per entry
+    extras: Dict[str, object] = field(default_factory=dict)   # what faster kernels plan on the host
+
+
+@dataclass
+class StepBatch:
+    entries: List[Entry]
+    stages: List[StageBatch]
+    n_wanted: int
+
+
+class _Packer:
+    """Collects int32 arrays, uploads them in one copy, hands back device views."""
+
+    def __init__(self):
+        self.parts: List[np.ndarray] = []
+        self.offsets: List[Tuple[int, Tuple[int, ...]]] = []
+        self.total = 0
+
+    def add(self, arr, shape=None) -> int:
+        a = np.ascontiguousarray(arr, dtype=np.int32).reshape(-1)
+        shape = tuple(shape) if shape is not None else (a.size,)
+        self.parts.append(a)
+        self.offsets.append((self.total, shape))
+        self.total += (a.size + 3) // 4 * 4          # keep every array 16-byte aligned
+        return len(self.offsets) - 1
+
+    def upload(self, device) -> List[torch.Tensor]:
+        host = torch.zeros(max(self.total, 4), dtype=torch.int32, pin_memory=(torch.device(device).type == "cuda"))
+        flat = host.numpy()
+        for a, (off, _) in zip(self.parts, self.offsets):
+            flat[off:off + a.size] = a
+        dev = host.to(device, non_blocking=True)
+        out = []
+        for a, (off, shape) in zip(self.parts, self.offsets):
+            out.append(dev[off:off + a.size].view(shape))
+        return out
+
+
+def build_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: Sequence[bool], cache, device,
+                     max_context: int) -> StepBatch:
+    """Row arrays for every stage of one step. `cache` is the CacheManager that already covers the new positions."""
+    n_seqs = len(entries)
+    pk = _Packer()
+    page_size = cache.page_size
+
+    # block tables: one line per entry, padded; shared by all stages
+    bt_ids = {}
+    for gname, g in cache.groups.items():
+        width = max(1, max(len(g.tables[e.slot]) for e in entries))
+        tab = np.zeros((n_seqs, width), dtype=np.int32)
+        for k, e in enumerate(entries):
+            t = g.tables[e.slot]
+            tab[k, :len(t)] = [p if p >= 0 else 0 for p in t]
+        bt_ids[gname] = pk.add(tab, tab.shape)
+    slots_id = pk.add([e.slot for e in entries])
+
+    plans = []
+    prev_rows: Optional[List[Tuple[int, int, int]]] = None
+    for j, lag in enumerate(lags):
+        tokens, positions, row_seq, cu = [], [], [], [0]
+        seq_rows = []
+        source, keep_src, keep_slot = [], [], []
+        for k, e in enumerate(entries):
+            s, n_tok = e.start, len(e.tokens)
+            end = s + n_tok
+            p0 = max(0, s - lag)
+            n = max(0, end - lag - p0)
+            off = len(e.tokens) - n
+            first_row = len(tokens)
+            if end > max_context:
+                raise ValueError(f"request in slot {e.slot} would reach position {end - 1}, "
+                                 f"beyond the model's context of {max_context}")
+            tokens.extend(int(t) for t in e.tokens[off:])
+            positions.extend(range(p0, p0 + n))
+            row_seq.extend([k] * n)
+            cu.append(len(tokens))
+            seq_rows.append((first_row, p0, n))
+            if has_source[j]:
+                pfirst, pp0, pn = prev_rows[k]
+                for p in range(p0, p0 + n):
+                    source.append(pfirst + (p - pp0) if p >= pp0 else -(e.slot + 1))
+                if pn > 0:
+                    keep_src.append(pfirst + pn - 1)
+                    keep_slot.append(e.slot)
+        ws = {}
+        for gname, g in cache.groups.items():
+            arr = np.empty(len(tokens), dtype=np.int32)
+            for k, e in enumerate(entries):
+                first_row, p0, n = seq_rows[k]
+                if n:
+                    p = np.arange(p0, p0 + n)
+                    arr[first_row:first_row + n] = np.asarray(g.tables[e.slot], dtype=np.int64)[p // page_size] \
+                        * page_size + p % page_size
+            ws[gname] = pk.add(arr)
+        want, valid = [], []
+        for k, e in enumerate(entries):
+            first_row, p0, n = seq_rows[k]
+            for i in e.want:
+                if not (0 <= i < len(e.tokens)):
+                    raise ValueError(f"want index {i} is outside the entry's {len(e.tokens)} tokens")
+                p = e.start + i - lag
+                ok = p >= p0 and n > 0
+                want.append(first_row + (p - p0) if ok else -1)
+                valid.append(ok)
+        plans.append(dict(
+            lag=lag, n_rows=len(tokens), tokens=pk.add(tokens), positions=pk.add(positions),
+            row_seq=pk.add(row_seq), cu=pk.add(cu), ws=ws,
+            source=pk.add(source) if has_source[j] else None,
+            keep_src=pk.add(keep_src) if has_source[j] else None,
+            keep_slot=pk.add(keep_slot) if has_source[j] else None,
+            keep_count=len(keep_src), want=pk.add(want), valid=valid, seq_rows=seq_rows,
+            max_kv=max([p0 + n for _, p0, n in seq_rows if n > 0] or [0]),
+            max_rows=max([n for _, _, n in seq_rows] or [0])))
+        prev_rows = seq_rows
+
+    dev = pk.upload(device)
+    tables = {g: dev[i] for g, i in bt_ids.items()}
+    stages = []
+    for pl in plans:
+        stages.append(StageBatch(
+            lag=pl["lag"], n_rows=pl["n_rows"], n_seqs=n_seqs, tokens=dev[pl["tokens"]],
+            positions=dev[pl["positions"]], row_seq=dev[pl["row_seq"]], cu_rows=dev[pl["cu"]],
+            seq_slots=dev[slots_id], write_slots={g: dev[i] for g, i in pl["ws"].items()}, block_tables=tables,
+            source_index=dev[pl["source"]] if pl["source"] is not None else None,
+            keep_source=dev[pl["keep_src"]] if pl["keep_src"] is not None else None,
+            keep_slot=dev[pl["keep_slot"]] if pl["keep_slot"] is not None else None,
+            keep_count=pl["keep_count"], want_index=dev[pl["want"]], want_valid=pl["valid"],
+            max_kv_len=pl["max_kv"], max_seq_rows=pl["max_rows"], seq_rows=pl["seq_rows"]))
+    return StepBatch(list(entries), stages, sum(len(e.want) for e in entries))

@@ -1,0 +1,166 @@
+"""The engine: a model, its cache, and the one step function that generation and replay both drive.
+
+`step` takes a batch of (request, its next tokens): portions of prompts beside single decoded tokens,
+cut anywhere. It runs only those tokens, as one batch, on top of what earlier steps left in the cache,
+and returns 32-bit logits at the places asked for.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import torch
+
+from .. import architectures  # noqa: F401  (registers the built-in architectures)
+from ..cache.manager import CacheManager, OutOfPages
+from ..config.model_config import ARCHITECTURES, load_config
+from ..weights.loader import load_tensors
+from .batch import Entry, build_step_batch
+from .model import Model
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def resolve_dtype(dtype):
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype {dtype!r}: use 'bfloat16' or 'float32'") from None
+
+
+@dataclass
+class StepOutput:
+    logits: torch.Tensor                         # [wanted, vocab] float32, in the order of entries and want
+    head_logits: Optional[List[torch.Tensor]]    # per prediction stage: [wanted, vocab]; rows not valid yet are NaN
+    head_valid: Optional[List[List[bool]]]
+
+
+class Engine:
+    def __init__(self, model_dir: Optional[str] = None, *, config=None, tensors=None, dtype="bfloat16",
+                 page_size: int = 16, max_tokens: Optional[int] = None, n_pages: Optional[int] = None,
+                 max_requests: int = 64, device="cuda:0", ops=None):
+        self.dtype = resolve_dtype(dtype)
+        if model_dir is not None:
+            config = load_config(model_dir)
+        if config is None:
+            raise ValueError("give a model folder or a configuration with tensors")
+        self.config = config
+        arch = ARCHITECTURES.get(config.architecture)
+        self.spec = arch.build_spec(config)
+        if tensors is None:
+            if model_dir is None:
+                raise ValueError("a configuration without a model folder needs its tensors")
+            tensors = load_tensors(model_dir, self.spec)
+        if ops is None:
+            from ..ops.hip_ops import HipOps
+            ops = HipOps(device, self.dtype)
+        self.ops = ops
+        self.device = ops.device
+        self.model = Model(self.spec, tensors, ops)
+        if n_pages is None:
+            if max_tokens is None:
+                raise ValueError("give the cache's size as max_tokens or n_pages")
+            n_pages = -(-int(max_tokens) // page_size)
+        self.page_size = page_size
+        self.cache = CacheManager(self.model.cache_needs(), page_size, n_pages, max_requests, self.dtype, self.device)
+        self.requests: Dict[Hashable, Tuple[int, int]] = {}      # id -> (slot, positions fed)
+
+    # ---- requests ------------------------------------------------------------------------------------
+    def open(self, rid: Hashable) -> None:
+        if rid in self.requests:
+            raise ValueError(f"request {rid!r} is already live")
+        self.requests[rid] = (self.cache.open_request(), 0)
+
+    def close(self, rid: Hashable) -> None:
+        slot, _ = self.requests.pop(rid)
+        self.cache.close_request(slot)
+
+    def fed(self, rid: Hashable) -> int:
+        return self.requests[rid][1]
+
+    def pages_to_grow(self, rid: Hashable, n_tokens: int) -> int:
+        """Most pages any group must take so that `rid` can be fed `n_tokens` more."""
+        slot, fed = self.requests[rid]
+        return max(self.cache.pages_needed(slot, fed + n_tokens).values(), default=0)
+
+    def free_pages(self) -> int:
+        return min(self.cache.free_pages().values(), default=0)
+
+    def total_pages(self) -> int:
+        return min(self.cache.total_pages().values(), default=0)
+
+    # ---- the step ------------------------------------------------------------------------------------
+    @torch.no_grad()
+    def step(self, entries: Sequence[Tuple[Hashable, Sequence[int], Sequence[int]]], heads: bool = False) -> StepOutput:
+        """entries: (request id, its next tokens, indices among them whose logits are wanted).
+
+        A request that is not live yet is opened. Raises OutOfPages, before anything is run or taken, if
+        the cache cannot hold the new tokens.
+        """
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        seen = set()
+        for rid, toks, _ in entries:
+            if rid in seen:
+                raise ValueError(f"request {rid!r} appears twice in one step")
+            seen.add(rid)
+            if len(toks) == 0:
+                raise ValueError(f"request {rid!r} brings no tokens")
+            for t in toks:
+                if not (0 <= int(t) < self.spec.vocab_size):
+                    raise ValueError(f"token {t} of request {rid!r} is outside the vocabulary of {self.spec.vocab_size}")
+        opened = []
+        for rid, _, _ in entries:
+            if rid not in self.requests:
+                self.open(rid)
+                opened.append(rid)
+        wants = {self.requests[rid][0]: self.requests[rid][1] + len(toks) for rid, toks, _ in entries}
+        too_long = [rid for rid, toks, _ in entries if self.requests[rid][1] + len(toks) > self.spec.max_context]
+        if too_long or not self.cache.can_grow(wants):
+            for rid in opened:
+                self.close(rid)
+            if too_long:
+                raise ValueError(f"request {too_long[0]!r} would pass the model's context of {self.spec.max_context}")
+            raise OutOfPages(f"the cache cannot take this step: it needs "
+                             f"{ {g: sum(grp.pages_for(s, n) for s, n in wants.items()) for g, grp in self.cache.groups.items()} } "
+                             f"pages, free are {self.cache.free_pages()}")
+        batch_entries = []
+        for rid, toks, want in entries:
+            slot, fed = self.requests[rid]
+            self.cache.grow(slot, fed + len(toks))
+            batch_entries.append(Entry(slot, fed, list(toks), list(want)))
+        step = build_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache, self.device,
+                                self.spec.max_context)
+        self.plan(step)
+        outs = self.model.forward(step, self.cache)
+        n = step.n_wanted
+        vocab = self.spec.vocab_size
+        if n:
+            logits = self.model.logits(outs[0].hidden, step.stages[0].want_index, n)
+        else:
+            logits = torch.empty(0, vocab, dtype=torch.float32, device=self.device)
+        head_logits = head_valid = None
+        if heads and len(outs) > 1:
+            head_logits, head_valid = [], []
+            for o in outs[1:]:
+                valid = o.batch.want_valid
+                if n and o.batch.n_rows and any(valid):
+                    idx = torch.clamp(o.batch.want_index[:n], min=0)
+                    lg = self.model.logits(o.hidden, idx, n)
+                    lg[~torch.tensor(valid, device=self.device)] = float("nan")
+                else:
+                    lg = torch.full((n, vocab), float("nan"), dtype=torch.float32, device=self.device)
+                head_logits.append(lg)
+                head_valid.append(list(valid))
+        for rid, toks, _ in entries:
+            slot, fed = self.requests[rid]
+            self.requests[rid] = (slot, fed + len(toks))
+            self.cache.release_behind(slot, fed + len(toks), self.model.max_lag)
+        return StepOutput(logits, head_logits, head_valid)
+
+    def plan(self, step) -> None:
+        """Host-side planning that the kernels of this ops object want for a step (none for the plain kernels)."""
+        planner = getattr(self.ops, "plan_step", None)
+        if planner is not None:
+            planner(step, self.cache)

@@ -1,0 +1,91 @@
+"""A model built from a spec of parts, and the pass that runs a step's rows through it.
+
+Nothing here knows an architecture: the spec says which layers exist, in which order each stage calls
+them, whose cache a call uses, where a stage's rows come from and which norm closes it.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..parts.base import ARRANGEMENTS, CallContext, Tensors, build_part, part_class, to_compute
+from ..parts.spec import ModelSpec, PagedKvNeed, StateNeed
+
+
+class StageOutput:
+    def __init__(self, hidden, batch):
+        self.hidden = hidden        # [rows, d_model], after the stage's closing norm
+        self.batch = batch
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], ops):
+        self.spec, self.ops = spec, ops
+        T = Tensors(tensors)
+        self.layers = [ARRANGEMENTS.get(ls.arrangement)(ls, T, ops) for ls in spec.layers]
+        self.inputs = [build_part(st.input, T, ops) for st in spec.stages]
+        self.out_norms = [build_part(st.out_norm, T, ops) for st in spec.stages]
+        emb = to_compute(ops, tensors[spec.embedding])
+        self.shared = {"embedding": emb,
+                       "lm_head": emb if spec.lm_head == spec.embedding else to_compute(ops, tensors[spec.lm_head])}
+        self.lags = [st.lag for st in spec.stages]
+        self.max_lag = max(self.lags)
+        self.reads_previous = [bool(getattr(part_class(st.input), "reads_previous", False)) for st in spec.stages]
+        if self.reads_previous and self.reads_previous[0]:
+            raise ValueError("the first stage cannot read a previous stage")
+        # cache keys: one per call unless the call names another's
+        self.call_keys: List[List[str]] = []
+        self.needs: Dict[str, object] = {}
+        for st in spec.stages:
+            keys = []
+            for i, call in enumerate(st.calls):
+                key = call.cache or f"{st.name}.{i}"
+                need = part_class(spec.layers[call.layer].mixer).cache_need(spec.layers[call.layer].mixer.params)
+                if call.writes_cache or key not in self.needs:
+                    if key in self.needs and self.needs[key] != need:
+                        raise ValueError(f"cache {key!r} is shared by layers that need different things: "
+                                         f"{self.needs[key]} and {need}")
+                    if need is not None:
+                        self.needs[key] = need
+                keys.append(key)
+            self.call_keys.append(keys)
+        self.state_keys: List[Optional[str]] = []
+        for st in spec.stages:
+            need = part_class(st.input).state_need(st.input.params)
+            key = (st.state_key or f"{st.name}.input") if need is not None else None
+            if key is not None:
+                self.needs[key] = need
+            self.state_keys.append(key)
+
+    def cache_needs(self) -> Dict[str, object]:
+        return dict(self.needs)
+
+    def forward(self, step, cache) -> List[StageOutput]:
+        """Run every stage over its rows; keys, values and state land in `cache`."""
+        outs: List[StageOutput] = []
+        prev = None
+        for j, st in enumerate(self.spec.stages):
+            b = step.stages[j]
+            state = cache.states.get(self.state_keys[j]) if self.state_keys[j] else None
+            x = self.inputs[j].forward(b, prev, self.shared, state)
+            if b.n_rows:
+                for i, call in enumerate(st.calls):
+                    key = self.call_keys[j][i]
+                    need = self.needs.get(key)
+                    ctx = CallContext(batch=b, writes_cache=call.writes_cache)
+                    if isinstance(need, PagedKvNeed):
+                        ctx.group = cache.group_of[key]
+                        ctx.plane = cache.groups[ctx.group].plane(key)
+                    elif isinstance(need, StateNeed):
+                        ctx.state = cache.states[key]
+                    x = self.layers[call.layer].forward(x, ctx)
+                x = self.out_norms[j](x)
+            prev = x
+            outs.append(StageOutput(x, b))
+        return outs
+
+    def logits(self, hidden, want_index, n):
+        """32-bit logits [n, vocab] of the rows `want_index` of `hidden` (reference main_models_new.py:225-226)."""
+        rows = self.ops.gather_rows(hidden, hidden, want_index[:n])
+        return self.ops.linear(rows, self.shared["lm_head"], out_dtype=torch.float32)

@@ -1,0 +1,345 @@
+"""The kernels as Python calls on torch tensors: what the parts and the engine compute with.
+
+Every method checks on the host that shapes, dtypes and strides are what the kernel and its grid assume,
+then launches on torch's current stream. There is no CPU path: without a GPU or without the compiled
+libraries construction fails. Matrix products in bfloat16 go to the library behind torch.matmul, as the
+reference's do (main_models_new.py:19-20); in 32-bit they go to the plain multiply-add kernel so that no
+reduced-precision matrix mode can take part.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
+
+
+class _Lib:
+    """One compiled library with typed entry points that raise on failure."""
+
+    def __init__(self, name: str, prefix: str, signatures: dict):
+        self.name = name
+        self.cdll = _build.load(name)
+        self._err = getattr(self.cdll, f"{prefix}_last_error")
+        self._err.restype = ctypes.c_char_p
+        for fn, argtypes in signatures.items():
+            f = getattr(self.cdll, fn)
+            f.argtypes = argtypes
+            f.restype = c_int
+            setattr(self, fn, self._wrap(f))
+
+    def _wrap(self, f):
+        def call(*args):
+            if f(*args) != 0:
+                raise KernelError(self._err().decode(errors="replace"))
+        return call
+
+
+_P, _I, _L, _F = c_void_p, c_int, c_long, c_float
+
+_SIGNATURES = {
+    "rowwise": ("tis_rowwise", {
+        "tis_rmsnorm": [_I, _P, _L, _P, _P, _L, _I, _I, _F, _P],
+        "tis_embedding": [_I, _P, _P, _P, _L, _I, _I, _P],
+        "tis_embedding_rmsnorm": [_I, _P, _P, _P, _P, _L, _I, _I, _F, _P],
+        "tis_gather_rows": [_I, _P, _L, _P, _L, _P, _P, _L, _I, _I, _P],
+        "tis_copy_rows": [_I, _P, _L, _P, _P, _L, _P, _I, _I, _P],
+        "tis_swiglu": [_I, _P, _L, _P, _L, _I, _I, _P],
+    }),
+    "rope_cache": ("tis_rope_cache", {
+        "tis_rope_write_kv": [_I, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    }),
+    "attention_generic": ("tis_attention_generic", {
+        "tis_attention_generic": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _F, _P],
+    }),
+    "gemm_plain": ("tis_gemm_plain", {
+        "tis_gemm_plain": [_I, _I, _P, _L, _P, _L, _P, _L, _P, _L, _I, _I, _I, _P],
+    }),
+    "sampling": ("tis_sampling", {
+        "tis_sample": [_P, _L, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P],
+        "tis_argmax": [_P, _L, _I, _I, _P, _P],
+    }),
+}
+
+_libs = {}
+
+
+def library(name: str) -> _Lib:
+    lib = _libs.get(name)
+    if lib is None:
+        prefix, sigs = _SIGNATURES[name]
+        lib = _libs[name] = _Lib(name, prefix, sigs)
+    return lib
+
+
+def _rows_view(t: torch.Tensor, what: str):
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{what}: expected a 2-d tensor with unit column stride, got shape {tuple(t.shape)} "
+                          f"strides {t.stride()}")
+    return t
+
+
+class HipOps:
+    """The operations of one engine instance: a device, a compute dtype, and the kernels for them."""
+
+    def __init__(self, device="cuda:0", dtype=torch.bfloat16):
+        if dtype not in _DT:
+            raise KernelError(f"unsupported compute dtype {dtype}; use torch.bfloat16 or torch.float32")
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: this engine runs on HIP kernels only and has no CPU path")
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.code = _DT[dtype]
+        self.rowwise = library("rowwise")
+        self.rope = library("rope_cache")
+        self.attn_generic = library("attention_generic")
+        self.gemm_plain = library("gemm_plain")
+        self.sampling = library("sampling")
+
+    # ---- helpers -------------------------------------------------------------------------------------
+    def _stream(self):
+        return c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _check(self, t: torch.Tensor, what: str, dtype=None):
+        dtype = dtype or self.dtype
+        if t.device != self.device and not (t.device.type == self.device.type and
+                                            (t.device.index or 0) == (self.device.index or 0)):
+            raise KernelError(f"{what}: tensor is on {t.device}, engine on {self.device}")
+        if t.dtype != dtype:
+            raise KernelError(f"{what}: dtype {t.dtype}, expected {dtype}")
+        return t
+
+    def _index(self, t: torch.Tensor, what: str, n: Optional[int] = None):
+        self._check(t, what, torch.int32)
+        if not t.is_contiguous():
+            raise KernelError(f"{what}: index tensor must be contiguous")
+        if n is not None and t.numel() < n:
+            raise KernelError(f"{what}: {t.numel()} entries for {n} rows")
+        return t
+
+    def empty(self, *shape, dtype=None):
+        return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)
+
+    # ---- row-wise ------------------------------------------------------------------------------------
+    def embedding(self, table, tokens, out=None):
+        self._check(table, "embedding table")
+        n = tokens.numel()
+        self._index(tokens, "tokens")
+        D = table.shape[1]
+        if out is None:
+            out = self.empty(n, D)
+        _rows_view(self._check(out, "embedding out"), "embedding out")
+        if out.shape[0] < n or out.shape[1] != D or not table.is_contiguous():
+            raise KernelError(f"embedding: out {tuple(out.shape)} does not fit {n} rows of {D}")
+        self.rowwise.tis_embedding(self.code, _ptr(table), _ptr(tokens), _ptr(out), out.stride(0), n, D,
+                                   self._stream())
+        return out
+
+    def rmsnorm(self, x, gain, eps: float, out=None):
+        _rows_view(self._check(x, "rmsnorm x"), "rmsnorm x")
+        self._check(gain, "rmsnorm gain", torch.float32)
+        n, D = x.shape
+        if gain.numel() != D or not gain.is_contiguous():
+            raise KernelError(f"rmsnorm: gain has {gain.numel()} entries for width {D}")
+        if out is None:
+            out = self.empty(n, D)
+        _rows_view(self._check(out, "rmsnorm out"), "rmsnorm out")
+        if tuple(out.shape) != (n, D):
+            raise KernelError(f"rmsnorm: out {tuple(out.shape)} vs x {tuple(x.shape)}")
+        self.rowwise.tis_rmsnorm(self.code, _ptr(x), x.stride(0), _ptr(gain), _ptr(out), out.stride(0), n, D,
+                                 float(eps), self._stream())
+        return out
+
+    def embedding_rmsnorm(self, table, tokens, gain, eps: float, out=None):
+        self._check(table, "embedding table")
+        self._check(gain, "rmsnorm gain", torch.float32)
+        self._index(tokens, "tokens")
+        n, D = tokens.numel(), table.shape[1]
+        if gain.numel() != D or not gain.is_contiguous() or not table.is_contiguous():
+            raise KernelError(f"embedding_rmsnorm: gain has {gain.numel()} entries for width {D}")
+        if out is None:
+            out = self.empty(n, D)
+        _rows_view(self._check(out, "embedding_rmsnorm out"), "embedding_rmsnorm out")
+        if out.shape[0] < n or out.shape[1] != D:
+            raise KernelError(f"embedding_rmsnorm: out {tuple(out.shape)} does not fit {n} rows of {D}")
+        self.rowwise.tis_embedding_rmsnorm(self.code, _ptr(table), _ptr(tokens), _ptr(gain), _ptr(out),
+                                           out.stride(0), n, D, float(eps), self._stream())
+        return out
+
+    def gather_rows(self, src, state, index, out=None):
+        """out[r] = src[index[r]] if index[r] >= 0 else state[-index[r]-1]."""
+        _rows_view(self._check(src, "gather src"), "gather src")
+        _rows_view(self._check(state, "gather state"), "gather state")
+        n = index.numel()
+        self._index(index, "gather index")
+        D = src.shape[1]
+        if state.shape[1] != D:
+            raise KernelError(f"gather_rows: src width {D}, state width {state.shape[1]}")
+        if out is None:
+            out = self.empty(n, D)
+        _rows_view(self._check(out, "gather out"), "gather out")
+        if out.shape[0] < n or out.shape[1] != D:
+            raise KernelError(f"gather_rows: out {tuple(out.shape)} does not fit {n} rows of {D}")
+        self.rowwise.tis_gather_rows(self.code, _ptr(src), src.stride(0), _ptr(state), state.stride(0), _ptr(index),
+                                     _ptr(out), out.stride(0), n, D, self._stream())
+        return out
+
+    def copy_rows(self, src, src_index, dst, dst_index):
+        """dst[dst_index[i]] = src[src_index[i]]."""
+        _rows_view(self._check(src, "copy src"), "copy src")
+        _rows_view(self._check(dst, "copy dst"), "copy dst")
+        n = src_index.numel()
+        self._index(src_index, "copy src_index")
+        self._index(dst_index, "copy dst_index", n)
+        if src.shape[1] != dst.shape[1]:
+            raise KernelError(f"copy_rows: widths {src.shape[1]} and {dst.shape[1]}")
+        self.rowwise.tis_copy_rows(self.code, _ptr(src), src.stride(0), _ptr(src_index), _ptr(dst), dst.stride(0),
+                                   _ptr(dst_index), n, src.shape[1], self._stream())
+
+    def swiglu(self, gu, out=None):
+        """out[:, f] = silu(gu[:, f]) * gu[:, F + f]."""
+        _rows_view(self._check(gu, "swiglu in"), "swiglu in")
+        n, F2 = gu.shape
+        if F2 % 2:
+            raise KernelError(f"swiglu: input width {F2} is odd")
+        F = F2 // 2
+        if out is None:
+            out = self.empty(n, F)
+        _rows_view(self._check(out, "swiglu out"), "swiglu out")
+        if tuple(out.shape) != (n, F):
+            raise KernelError(f"swiglu: out {tuple(out.shape)} for {n} rows of {F}")
+        self.rowwise.tis_swiglu(self.code, _ptr(gu), gu.stride(0), _ptr(out), out.stride(0), n, F, self._stream())
+        return out
+
+    # ---- matrix products -----------------------------------------------------------------------------
+    def linear(self, x, w, residual=None, out_dtype=None):
+        """x[M,K] . w[N,K]^T (+ residual[M,N]); `out_dtype` float32 gives 32-bit results from bfloat16 inputs."""
+        _rows_view(self._check(x, "linear x"), "linear x")
+        self._check(w, "linear w")
+        out_dtype = out_dtype or self.dtype
+        M, K = x.shape
+        if w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+            raise KernelError(f"linear: x {tuple(x.shape)} against w {tuple(w.shape)} (w is [out, in], contiguous)")
+        N = w.shape[0]
+        if residual is not None:
+            _rows_view(self._check(residual, "linear residual", out_dtype), "linear residual")
+            if tuple(residual.shape) != (M, N):
+                raise KernelError(f"linear: residual {tuple(residual.shape)} for result {(M, N)}")
+        if self.dtype == torch.float32:
+            out = self.empty(M, N, dtype=torch.float32)
+            self.gemm_plain.tis_gemm_plain(0, 0, _ptr(x), x.stride(0), _ptr(w), K, _ptr(residual),
+                                           residual.stride(0) if residual is not None else 0, _ptr(out), N, M, N, K,
+                                           self._stream())
+            return out
+        return self._linear_bf16(x, w, residual, out_dtype)
+
+    def _linear_bf16(self, x, w, residual, out_dtype):
+        if out_dtype == torch.float32:
+            out = torch.matmul(x, w.t()).float()
+            if residual is not None:
+                out += residual
+            return out
+        if residual is not None:
+            return torch.addmm(residual, x, w.t())
+        return torch.matmul(x, w.t())
+
+    # ---- position encoding + cache write, attention --------------------------------------------------
+    def rope_write_kv(self, qkv, positions, write_slots, table, plane, n_heads, n_kv_heads, head_dim, page_size,
+                      interleaved=False, write_cache=True):
+        _rows_view(self._check(qkv, "qkv"), "qkv")
+        n = qkv.shape[0]
+        if qkv.shape[1] != (n_heads + 2 * n_kv_heads) * head_dim:
+            raise KernelError(f"rope_write_kv: row width {qkv.shape[1]} is not (heads {n_heads} + 2 x kv heads "
+                              f"{n_kv_heads}) x head size {head_dim}")
+        self._index(positions, "positions", n)
+        if table is not None:
+            self._check(table, "rotary table", torch.float32)
+            if table.dim() != 3 or table.shape[1] != head_dim // 2 or table.shape[2] != 2 or not table.is_contiguous():
+                raise KernelError(f"rope_write_kv: table {tuple(table.shape)} for head size {head_dim}")
+        if write_cache:
+            self._index(write_slots, "write_slots", n)
+            self._check_plane(plane, n_kv_heads, head_dim, page_size)
+        self.rope.tis_rope_write_kv(self.code, _ptr(qkv), qkv.stride(0), _ptr(positions),
+                                    _ptr(write_slots if write_cache else None), _ptr(table),
+                                    _ptr(plane if write_cache else None), n, n_heads, n_kv_heads, head_dim, page_size,
+                                    int(bool(interleaved)), int(bool(write_cache)), self._stream())
+
+    def _check_plane(self, plane, n_kv_heads, head_dim, page_size):
+        self._check(plane, "cache plane")
+        if plane.dim() != 5 or tuple(plane.shape[1:]) != (2, n_kv_heads, page_size, head_dim) or \
+                not plane.is_contiguous():
+            raise KernelError(f"cache plane {tuple(plane.shape)} is not [pages, 2, {n_kv_heads}, {page_size}, "
+                              f"{head_dim}] contiguous")
+
+    def paged_attention(self, q, plane, batch, group, n_heads, n_kv_heads, head_dim, window=0, scale=None):
+        """Attention of the rows in `batch` over the cache plane; `q` is [rows, heads*head_dim] (a strided view is fine).
+
+        `batch` brings positions, row_seq and the group's block tables; `group` names the page group.
+        """
+        _rows_view(self._check(q, "q"), "q")
+        n = q.shape[0]
+        page_size = plane.shape[3]
+        self._check_plane(plane, n_kv_heads, head_dim, page_size)
+        if q.shape[1] != n_heads * head_dim:
+            raise KernelError(f"attention: q width {q.shape[1]} is not heads {n_heads} x head size {head_dim}")
+        tables = batch.block_tables[group]
+        self._check(tables, "block tables", torch.int32)
+        if tables.dim() != 2 or tables.stride(1) != 1:
+            raise KernelError(f"attention: block tables {tuple(tables.shape)} must be 2-d")
+        self._index(batch.positions, "positions", n)
+        self._index(batch.row_seq, "row_seq", n)
+        if batch.max_kv_len > tables.shape[1] * page_size:
+            raise KernelError(f"attention: a row sees {batch.max_kv_len} keys but block tables cover "
+                              f"{tables.shape[1] * page_size}")
+        if scale is None:
+            scale = head_dim ** -0.5
+        out = self.empty(n, n_heads * head_dim)
+        self.attn_generic.tis_attention_generic(
+            self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
+            _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, head_dim, page_size, int(window),
+            float(scale), self._stream())
+        return out
+
+    # ---- sampling ------------------------------------------------------------------------------------
+    def argmax(self, logits):
+        _rows_view(self._check(logits, "logits", torch.float32), "logits")
+        n, V = logits.shape
+        out = torch.empty(n, dtype=torch.int32, device=self.device)
+        self.sampling.tis_argmax(_ptr(logits), logits.stride(0), n, V, _ptr(out), self._stream())
+        return out
+
+    def sample(self, logits, temperature, top_k, top_p, rep_penalty, uniform, ctx_tokens=None, ctx_offsets=None):
+        """One token per row of 32-bit logits; per-row parameters are device tensors of length rows."""
+        _rows_view(self._check(logits, "logits", torch.float32), "logits")
+        n, V = logits.shape
+        for t, what, dt in ((temperature, "temperature", torch.float32), (top_p, "top_p", torch.float32),
+                            (uniform, "uniform", torch.float32), (top_k, "top_k", torch.int32)):
+            self._check(t, what, dt)
+            if t.numel() != n or not t.is_contiguous():
+                raise KernelError(f"sample: {what} has {t.numel()} entries for {n} rows")
+        if rep_penalty is not None:
+            self._check(rep_penalty, "rep_penalty", torch.float32)
+            if rep_penalty.numel() != n:
+                raise KernelError(f"sample: rep_penalty has {rep_penalty.numel()} entries for {n} rows")
+        if ctx_tokens is not None:
+            self._index(ctx_tokens, "ctx_tokens")
+            self._index(ctx_offsets, "ctx_offsets", n + 1)
+        work = torch.empty(n, V, dtype=torch.float32, device=self.device)
+        out = torch.empty(n, dtype=torch.int32, device=self.device)
+        self.sampling.tis_sample(_ptr(logits), logits.stride(0), _ptr(work), n, V, _ptr(temperature), _ptr(top_k),
+                                 _ptr(top_p), _ptr(rep_penalty), _ptr(ctx_tokens), _ptr(ctx_offsets), _ptr(uniform),
+                                 _ptr(out), self._stream())
+        return out

@@ -1,0 +1,57 @@
+"""Attention mixers."""
+from __future__ import annotations
+
+import torch
+
+from .base import MIXERS, build_part, to_compute
+from .spec import PagedKvNeed
+
+
+@MIXERS.register("gqa_attention")
+class GqaAttention:
+    """Grouped-query attention over a paged cache.
+
+    q = x.Wq, [k|v] = x.Wkv, rotary on q and k, keys and values written into the call's cache plane before
+    any row attends, then every row at position p attends the keys [0, p] (or the last `window`) of its
+    own request, query head h using key/value head h // group_size; out = attn.Wo (+ residual)
+    (reference main_models_new.py:96-136; paged_attention_kernels.py:49).
+
+    params: d_model, n_heads, n_kv_heads, head_dim, window (0: all keys), position (a PartSpec).
+    tensors: q (d_model, n_heads*head_dim), kv (d_model, 2*n_kv_heads*head_dim) with the key columns first,
+    o (n_heads*head_dim, d_model); all stored [in, out] as the reference applies them (x @ W).
+    """
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        d, nh, nkv, hd = params["d_model"], params["n_heads"], params["n_kv_heads"], params["head_dim"]
+        return {"q": (d, nh * hd), "kv": (d, 2 * nkv * hd), "o": (nh * hd, d)}
+
+    @classmethod
+    def cache_need(cls, params):
+        return PagedKvNeed(params["n_kv_heads"], params["head_dim"], int(params.get("window", 0)))
+
+    def __init__(self, spec, tensors, ops):
+        p = spec.params
+        self.ops = ops
+        self.n_heads, self.n_kv_heads, self.head_dim = int(p["n_heads"]), int(p["n_kv_heads"]), int(p["head_dim"])
+        if self.n_heads % self.n_kv_heads:
+            raise ValueError(f"{self.n_heads} query heads are not a multiple of {self.n_kv_heads} key/value heads")
+        self.window = int(p.get("window", 0))
+        self.scale = float(p.get("scale", self.head_dim ** -0.5))
+        pos = p["position"]
+        self.position = build_part(pos, tensors, ops)
+        # one projection for q, k and v: rows of the [out, in] matrix are q heads, then k heads, then v heads
+        self.w_qkv = to_compute(ops, torch.cat((tensors.of(spec, "q"), tensors.of(spec, "kv")), dim=1).t())
+        self.w_o = to_compute(ops, tensors.of(spec, "o").t())
+        self.q_width = self.n_heads * self.head_dim
+
+    def forward(self, x, ctx, residual=None):
+        ops, b = self.ops, ctx.batch
+        qkv = ops.linear(x, self.w_qkv)
+        table, interleaved = self.position.rotary()
+        page_size = ctx.plane.shape[3]
+        ops.rope_write_kv(qkv, b.positions, b.write_slots[ctx.group], table, ctx.plane, self.n_heads,
+                          self.n_kv_heads, self.head_dim, page_size, interleaved, ctx.writes_cache)
+        attn = ops.paged_attention(qkv[:, :self.q_width], ctx.plane, b, ctx.group, self.n_heads, self.n_kv_heads,
+                                   self.head_dim, self.window, self.scale)
+        return ops.linear(attn, self.w_o, residual=residual)

@@ -1,0 +1,100 @@
+"""Registries of part kinds and the interfaces the engine expects of them.
+
+A part is built from a `PartSpec` (its sizes and constants), the tensors it named, and an `ops` object
+that carries the kernels, the device and the compute dtype. No part is told which model it belongs to.
+
+Interfaces
+----------
+every part class
+    tensor_shapes(params) -> {local key: shape}        classmethod; what it wants from the weight file
+    __init__(spec, tensors, ops)                       tensors.of(spec, key) -> the CPU tensor as stored;
+                                                       nested parts are built with build_part(sub_spec, tensors, ops)
+
+norm            __call__(x) -> y                       rows in, rows out
+position        rotary() -> (table | None, interleaved)   a table of (cos, sin) per position and pair for
+                                                       mixers that rotate queries and keys; and
+                on_embedding(x, batch) -> x            a hook for encodings that act on the embedded rows
+mixer           cache_need(params) -> PagedKvNeed | StateNeed | None      classmethod
+                forward(x, ctx, residual=None) -> y    x: normed rows; ctx: CallContext; adds `residual` if given
+feed-forward    forward(x, residual=None) -> y
+arrangement     __init__(layer_spec, parts...), forward(x, ctx) -> x      how norm, mixer and feed-forward are wired
+stage input     state_need(params) -> StateNeed | None classmethod
+                forward(batch, previous_output, previous_batch, shared, state) -> rows
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Optional
+
+from ..config.registry import Registry
+
+MIXERS: Registry = Registry("mixer")
+FEED_FORWARDS: Registry = Registry("feed-forward")
+NORMS: Registry = Registry("norm")
+POSITION_ENCODINGS: Registry = Registry("position encoding")
+ARRANGEMENTS: Registry = Registry("block arrangement")
+STAGE_INPUTS: Registry = Registry("stage input")
+
+
+@dataclass
+class CallContext:
+    """What one layer call sees of the step: the rows' metadata and the cache that belongs to the call."""
+    batch: Any                       # engine.batch.StageBatch
+    group: Optional[str] = None      # page group of the call's cache, for paged needs
+    plane: Any = None                # [pages, 2, kv heads, page size, head size] for paged needs
+    state: Any = None                # [max requests, *shape] for state needs
+    writes_cache: bool = True
+
+
+class Tensors:
+    """The loaded tensors by their names in the file; a part asks for its own by local key."""
+
+    def __init__(self, by_name):
+        self.by_name = by_name
+
+    def of(self, spec, key):
+        try:
+            return self.by_name[spec.tensors[key]]
+        except KeyError:
+            raise KeyError(f"part {spec.kind!r} asks for tensor {key!r} -> {spec.tensors.get(key)!r}, "
+                           f"which was not loaded") from None
+
+
+REGISTRIES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "position": POSITION_ENCODINGS,
+              "stage_input": STAGE_INPUTS}
+
+
+def part_class(spec):
+    try:
+        registry = REGISTRIES[spec.role]
+    except KeyError:
+        raise KeyError(f"unknown part role {spec.role!r}; known: {', '.join(sorted(REGISTRIES))}") from None
+    return registry.get(spec.kind)
+
+
+def build_part(spec, tensors, ops):
+    return part_class(spec)(spec, tensors, ops)
+
+
+def expected_tensors(spec):
+    """{tensor name in the file: shape} of a part and of the parts nested in its params."""
+    out = {}
+    shapes = part_class(spec).tensor_shapes(spec.params)
+    for key, shape in shapes.items():
+        if key not in spec.tensors:
+            raise KeyError(f"part {spec.kind!r} needs a tensor name for {key!r}")
+        out[spec.tensors[key]] = tuple(int(s) for s in shape)
+    for v in spec.params.values():
+        if hasattr(v, "role") and hasattr(v, "kind"):
+            out.update(expected_tensors(v))
+    return out
+
+
+def to_compute(ops, t):
+    """A stored matrix as the kernels take it: on the device, in the compute dtype."""
+    return t.to(device=ops.device, dtype=ops.dtype).contiguous()
+
+
+def to_gain(ops, t):
+    """A stored 1-d gain on the device in 32-bit (widening bfloat16 is exact)."""
+    return t.to(device=ops.device, dtype=__import__("torch").float32).contiguous()

@@ -1,0 +1,19 @@
+"""Arrangements: how a block wires its norms, its mixer and its feed-forward."""
+from __future__ import annotations
+
+from .base import ARRANGEMENTS, build_part
+
+
+@ARRANGEMENTS.register("prenorm_residual")
+class PreNormResidual:
+    """x = x + mixer(norm_a(x)); x = x + feed_forward(norm_f(x))   (reference main_models_new.py:146-152)."""
+
+    def __init__(self, layer_spec, tensors, ops):
+        self.mixer_norm = build_part(layer_spec.mixer_norm, tensors, ops)
+        self.mixer = build_part(layer_spec.mixer, tensors, ops)
+        self.ffn_norm = build_part(layer_spec.feed_forward_norm, tensors, ops)
+        self.ffn = build_part(layer_spec.feed_forward, tensors, ops)
+
+    def forward(self, x, ctx):
+        x = self.mixer.forward(self.mixer_norm(x), ctx, residual=x)
+        return self.ffn.forward(self.ffn_norm(x), residual=x)

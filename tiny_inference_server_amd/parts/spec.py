@@ -1,0 +1,83 @@
+"""Plain data that describes a model as an arrangement of parts.
+
+An architecture turns its configuration into a `ModelSpec`; the engine builds
+and runs the spec and never asks which architecture it came from.
+
+* `PartSpec`      one part: its role and kind (a registry and a name in it), its sizes and
+                  constants, and the full names of the tensors it owns.
+* `LayerSpec`     one block: an arrangement kind and the parts it arranges.
+* `LayerCall`     one entry of the run order: which layer runs and whose cache it uses.
+* `StageSpec`     one pass over the rows of a step: where its input comes from,
+                  the ordered calls, the closing norm.  A stage with `lag` j runs
+                  at positions j behind the tokens that the step brings.
+* `ModelSpec`     the layers, the stages and the shared tables.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Mapping, Optional, Tuple
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    role: str                     # which registry `kind` is looked up in: "norm", "position", "mixer",
+                                  # "feed_forward" or "stage_input"
+    kind: str
+    params: Mapping[str, Any] = field(default_factory=dict)    # sizes, constants, nested PartSpecs
+    tensors: Mapping[str, str] = field(default_factory=dict)   # local key -> tensor name in the file
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    arrangement: str              # block arrangement kind, e.g. "prenorm_residual"
+    mixer: PartSpec
+    mixer_norm: PartSpec
+    feed_forward: PartSpec
+    feed_forward_norm: PartSpec
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    layer: int                        # index into ModelSpec.layers
+    cache: Optional[str] = None       # cache key; None: a key of this call's own
+    writes_cache: bool = True         # False: only reads what the owner of `cache` wrote
+
+
+@dataclass(frozen=True)
+class StageSpec:
+    name: str
+    lag: int                          # rows of this stage sit `lag` positions behind the step's tokens
+    input: PartSpec                   # "token_embedding" or "fuse_previous_stage"
+    calls: Tuple[LayerCall, ...]
+    out_norm: PartSpec
+    state_key: Optional[str] = None   # cache key of the input part's per-request state, if it has one
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    d_model: int
+    vocab_size: int
+    max_context: int
+    layers: Tuple[LayerSpec, ...]
+    stages: Tuple[StageSpec, ...]
+    embedding: str                    # tensor name of the token table (vocab, d_model)
+    lm_head: str                      # tensor name of the output table (vocab, d_model); the same name when tied
+    eos_token_id: int = -1
+    ignorable: Tuple[str, ...] = ()   # glob patterns of derived buffers a file may also hold
+
+
+# What a part needs from the cache manager --------------------------------------------------
+
+@dataclass(frozen=True)
+class PagedKvNeed:
+    """Keys and values of every position (window 0) or of the last `window` positions."""
+    n_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A block of fixed size for each live request."""
+    shape: Tuple[int, ...]
+    dtype: str = "compute"            # "compute": the engine's dtype; or "float32" / "int32"

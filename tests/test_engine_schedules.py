@@ -1,0 +1,122 @@
+"""The engine against the plain implementation under every way of cutting and batching the same requests.
+
+The same tests run twice: on the GPU with the HIP kernels (marked gpu), in 32-bit and in bfloat16, and on
+the CPU with the plain torch stand-ins for the kernels (tests/torch_ops.py), which checks the step function,
+the batch builder and the cache without a GPU. Tolerances are fixed: 2e-5 of the logits' scale in 32-bit,
+2e-2 in bfloat16 (bfloat16 keeps 8 bits; the measured error of a correct run is about a fifth of that).
+"""
+import pytest
+import torch
+
+import helpers as H
+from tiny_inference_server_amd.engine import Engine
+
+TOL = {"float32": 2e-5, "bfloat16": 2e-2}
+
+
+def backends():
+    return [pytest.param("hip", marks=pytest.mark.gpu), pytest.param("torch", marks=[])]
+
+
+def make_engine(name, dtype, backend, max_tokens, max_requests=4):
+    folder = H.model_folder(name, "float32" if dtype == "float32" else "bfloat16")
+    ops = None
+    if backend == "torch":
+        from torch_ops import TorchOps
+        ops = TorchOps(dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    eng = Engine(folder, dtype=dtype, page_size=H.TINY[name]["page_size"], max_tokens=max_tokens,
+                 max_requests=max_requests, ops=ops)
+    return folder, eng
+
+
+def requests_for(name, lengths, seed):
+    vocab = H.TINY[name]["cfg"].vocab_size
+    return {f"r{i}": H.random_ids(vocab, n, seed * 100 + i) for i, n in enumerate(lengths)}
+
+
+def scale_of(folder, reqs):
+    return max(1.0, max(H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values()))
+
+
+CASES = [("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16"), ("C", "bfloat16"),
+         ("D", "bfloat16"), ("D", "float32")]
+
+
+@pytest.mark.parametrize("backend", backends())
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_whole_requests(name, dtype, backend):
+    reqs = requests_for(name, [5, 17, 33, 1, 2, 70], seed=1)
+    folder, eng = make_engine(name, dtype, backend, max_tokens=128)
+    main, heads = H.run_trace(eng, H.whole_trace(reqs))
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.parametrize("backend", backends())
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_prefill_then_decode_one_by_one(name, dtype, backend):
+    reqs = requests_for(name, [75, 40, 33], seed=2)
+    folder, eng = make_engine(name, dtype, backend, max_tokens=128)
+    main, heads = H.run_trace(eng, H.tail_decode_trace(reqs, tail=32))
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.parametrize("backend", backends())
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_portions_of_changing_size(name, dtype, backend):
+    reqs = requests_for(name, [97, 50], seed=3)
+    folder, eng = make_engine(name, dtype, backend, max_tokens=128)
+    main, heads = H.run_trace(eng, H.portions_trace(reqs, seed=1))
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.parametrize("backend", backends())
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_mixed_batches_with_page_reuse(name, dtype, backend):
+    lengths = [50, 64, 37, 90, 18, 70, 45, 3, 66, 29]
+    reqs = requests_for(name, lengths, seed=4)
+    steps, peak = H.mixed_trace(reqs, max_live=4, seed=5)
+    # so few pages that finished requests' pages must be handed out again
+    folder, eng = make_engine(name, dtype, backend, max_tokens=peak)
+    assert sum(-(-n // 64) * 64 for n in lengths) > 2 * peak
+    main, heads = H.run_trace(eng, steps)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.parametrize("backend", backends())
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16")])
+def test_first_tokens_and_long_decoding(name, dtype, backend):
+    """One token at a time from the very first position: the heads start late, every page edge is crossed."""
+    n = 150 if name == "A" else 120
+    reqs = requests_for(name, [n], seed=6)
+    folder, eng = make_engine(name, dtype, backend, max_tokens=192)
+    ids = reqs["r0"]
+    steps = [{"step": p, "entries": [{"id": "r0", "tokens": [ids[p]], "want": [0]}],
+              "end": ["r0"] if p == n - 1 else []} for p in range(n)]
+    main, heads = H.run_trace(eng, steps)
+    assert len(main) == n
+    M = eng.config.mtp_heads
+    for hi in range(M):
+        assert all(("r0", hi, p) in heads for p in range(n - 1 - hi))
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), M)
+
+
+@pytest.mark.parametrize("backend", backends())
+def test_all_schedules_agree_with_each_other(backend):
+    """The same (request, position) under four schedules: differences stay within rounding of 32-bit sums."""
+    name, dtype = "B", "float32"
+    reqs = requests_for(name, [61, 44], seed=7)
+    outs = []
+    for trace in (H.whole_trace(reqs), H.tail_decode_trace(reqs, 32), H.portions_trace(reqs, 2),
+                  H.mixed_trace(reqs, 2, 3)[0]):
+        folder, eng = make_engine(name, dtype, backend, max_tokens=128)
+        outs.append(H.run_trace(eng, trace)[0])
+    for other in outs[1:]:
+        assert other.keys() == outs[0].keys()
+        worst = max((other[k] - outs[0][k]).abs().max().item() for k in other)
+        assert worst <= 2e-5

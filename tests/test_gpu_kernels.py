@@ -1,0 +1,294 @@
+"""Each HIP kernel alone against its plain torch reference (tests/torch_ops.py), at sizes other than the engine's
+tiny configurations: widths and vocabularies that are no power of two, odd head counts and groups, page edges."""
+import math
+import random
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from torch_ops import TorchOps
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+@pytest.fixture(scope="module")
+def ops_for():
+    from tiny_inference_server_amd.ops.hip_ops import HipOps
+    made = {}
+
+    def get(dtype):
+        if dtype not in made:
+            made[dtype] = HipOps("cuda:0", dtype)
+        return made[dtype]
+    return get
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (scale * torch.randn(shape, generator=g)).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,D", [(1, 8), (7, 1536), (33, 1000), (3, 5000)])
+def test_rmsnorm(ops_for, dtype, rows, D):
+    ops, ref = ops_for(dtype), TorchOps(dtype=dtype)
+    x = rnd((rows, D), dtype, 1, 3.0)
+    x[0] = 0                                   # an all-zero row gives 0, not NaN: eps sits outside the root
+    gain = 1 + 0.1 * rnd((D,), torch.float32, 2)
+    got = ops.rmsnorm(x.cuda(), gain.cuda(), 2e-8).cpu()
+    assert torch.isfinite(got).all() and (got[0] == 0).all()
+    torch.testing.assert_close(got.float(), ref.rmsnorm(x, gain, 2e-8).float(), **tol(dtype))
+    # strided input and output: the middle columns of a wider buffer
+    wide = rnd((rows, 2 * D), dtype, 3).cuda()
+    out = torch.zeros(rows, 2 * D, dtype=dtype, device="cuda")
+    ops.rmsnorm(wide[:, D:], gain.cuda(), 1e-5, out=out[:, :D])
+    torch.testing.assert_close(out[:, :D].cpu().float(), ref.rmsnorm(wide[:, D:].cpu(), gain, 1e-5).float(), **tol(dtype))
+    assert (out[:, D:] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_and_fused_norm_and_row_moves(ops_for, dtype):
+    ops, ref = ops_for(dtype), TorchOps(dtype=dtype)
+    V, D, n = 777, 200, 19
+    table = rnd((V, D), dtype, 4)
+    toks = torch.tensor([random.Random(5).randrange(V) for _ in range(n)], dtype=torch.int32)
+    gain = 1 + 0.1 * rnd((D,), torch.float32, 6)
+    assert torch.equal(ops.embedding(table.cuda(), toks.cuda()).cpu(), table[toks.long()])
+    out = torch.zeros(n, 2 * D, dtype=dtype, device="cuda")
+    ops.embedding_rmsnorm(table.cuda(), toks.cuda(), gain.cuda(), 1e-6, out=out[:, D:])
+    torch.testing.assert_close(out[:, D:].cpu().float(), ref.embedding_rmsnorm(table, toks, gain, 1e-6).float(), **tol(dtype))
+    # gather from rows or from state, then keep rows in state
+    src, state = rnd((n, D), dtype, 7), rnd((6, D), dtype, 8)
+    index = torch.tensor([3, -1, 0, -6, 18, 18, -2], dtype=torch.int32)
+    got = ops.gather_rows(src.cuda(), state.cuda(), index.cuda()).cpu()
+    assert torch.equal(got, ref.gather_rows(src, state, index))
+    st_gpu = state.cuda()
+    ops.copy_rows(src.cuda(), torch.tensor([4, 9], dtype=torch.int32).cuda(), st_gpu,
+                  torch.tensor([5, 0], dtype=torch.int32).cuda())
+    want = state.clone(); want[5] = src[4]; want[0] = src[9]
+    assert torch.equal(st_gpu.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,F", [(1, 176), (9, 4096), (5, 1001)])
+def test_swiglu(ops_for, dtype, rows, F):
+    ops, ref = ops_for(dtype), TorchOps(dtype=dtype)
+    gu = rnd((rows, 2 * F), dtype, 9, 2.0)
+    gu[:, 3] = 0                               # a zero gate gives a zero output whatever the other half holds
+    got = ops.swiglu(gu.cuda()).cpu()
+    assert (got[:, 3] == 0).all()
+    torch.testing.assert_close(got.float(), ref.swiglu(gu).float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 1000, 96), (70, 130, 257), (64, 2304, 1536), (3, 515, 512)])
+def test_linear(ops_for, dtype, M, N, K):
+    ops = ops_for(dtype)
+    x, w, res = rnd((M, K), dtype, 10), rnd((N, K), dtype, 11, K ** -0.5), rnd((M, N), dtype, 12)
+    want = x.double() @ w.double().t()
+    t = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(ops.linear(x.cuda(), w.cuda()).cpu().double(), want, **t)
+    torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), residual=res.cuda()).cpu().double(), want + res.double(), **t)
+    lg = ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32)
+    assert lg.dtype == torch.float32
+    torch.testing.assert_close(lg.cpu().double(), want, **t)
+
+
+def test_linear_32bit_is_true_32bit(ops_for):
+    """Products of numbers that need 24 bits: a reduced-precision matrix mode (tf32-like, bf16 x3) would lose them."""
+    ops = ops_for(torch.float32)
+    K = 512
+    x = (1 + torch.arange(K, dtype=torch.float64) * 2.0 ** -20).float().view(1, K)
+    w = (1 - torch.arange(K, dtype=torch.float64) * 2.0 ** -21).float().view(1, K)
+    want = (x.double() * w.double()).sum().item()
+    got = ops.linear(x.cuda(), w.cuda()).item()
+    assert abs(got - want) / want < 3e-7
+
+
+def make_paged(kv_lens, n_kv, hd, page_size, dtype, seed, shuffle=True):
+    """Keys and values of several requests scattered over shuffled pages (reference test_gqa_paged.py:15-28)."""
+    n_pages = sum(-(-L // page_size) for L in kv_lens) + 3
+    ids = list(range(n_pages))
+    if shuffle:
+        random.Random(seed).shuffle(ids)
+    # unused slots hold huge values: a kernel that reads a masked slot shows it
+    plane = torch.full((n_pages, 2, n_kv, page_size, hd), 3e4, dtype=dtype)
+    tables, ks, vs = [], [], []
+    width = max(-(-L // page_size) for L in kv_lens)
+    for i, L in enumerate(kv_lens):
+        k, v = rnd((L, n_kv, hd), dtype, seed + 10 * i), rnd((L, n_kv, hd), dtype, seed + 10 * i + 1)
+        pages = [ids.pop() for _ in range(-(-L // page_size))]
+        for j in range(L):
+            plane[pages[j // page_size], 0, :, j % page_size] = k[j]
+            plane[pages[j // page_size], 1, :, j % page_size] = v[j]
+        tables.append(pages + [0] * (width - len(pages)))
+        ks.append(k); vs.append(v)
+    return plane, torch.tensor(tables, dtype=torch.int32), ks, vs
+
+
+def dense_reference(q, k, v, group, pos, window=0):
+    """One row: query heads [NH, hd] against keys [0, pos] by library attention on repeated kv heads
+    (the reference's own oracle: test_gqa_paged.py:39-44)."""
+    lo = max(0, pos - window + 1) if window else 0
+    kq = k[lo:pos + 1].double().repeat_interleave(group, dim=1).transpose(0, 1)     # [NH, keys, hd]
+    vq = v[lo:pos + 1].double().repeat_interleave(group, dim=1).transpose(0, 1)
+    return torch.nn.functional.scaled_dot_product_attention(q.double()[:, None, :], kq, vq)[:, 0, :]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,page_size,kv_lens", [
+    (8, 2, 64, 16, [37, 512, 2000]),           # the reference's case: test_gqa_paged.py:11-17
+    (3, 1, 32, 8, [1, 9, 24, 40]),
+    (6, 3, 48, 16, [16, 17, 300]),
+    (12, 3, 128, 16, [4096, 130]),
+    (5, 5, 8, 4, [3, 1100]),
+    (4, 1, 256, 32, [65]),
+])
+def test_paged_attention_single_rows(ops_for, dtype, n_heads, n_kv, hd, page_size, kv_lens):
+    """Decode-like rows: the last position of several requests with scattered pages."""
+    ops = ops_for(dtype)
+    group = n_heads // n_kv
+    plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page_size, dtype, seed=20)
+    B = len(kv_lens)
+    q = rnd((B, n_heads * hd), dtype, 21)
+    batch = SimpleNamespace(positions=torch.tensor([L - 1 for L in kv_lens], dtype=torch.int32).cuda(),
+                            row_seq=torch.arange(B, dtype=torch.int32).cuda(),
+                            block_tables={"g": tables.cuda()}, max_kv_len=max(kv_lens), extras={},
+                            n_rows=B, max_seq_rows=1, seq_rows=[(i, kv_lens[i] - 1, 1) for i in range(B)])
+    got = ops.paged_attention(q.cuda(), plane.cuda(), batch, "g", n_heads, n_kv, hd).cpu()
+    t = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    for i, L in enumerate(kv_lens):
+        want = dense_reference(q[i].view(n_heads, hd), ks[i], vs[i], group, L - 1)
+        torch.testing.assert_close(got[i].view(n_heads, hd).double(), want, **t)
+    if group > 1 and n_kv > 1:
+        # negative control (reference test_gqa_paged.py:50-53): the wrong head mapping must not match
+        bad = dense_reference(q[0].view(n_heads, hd), ks[0].flip(1), vs[0].flip(1), group, kv_lens[0] - 1)
+        assert not torch.allclose(got[0].view(n_heads, hd).double(), bad, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,page_size", [(4, 2, 64, 16), (3, 1, 32, 8), (12, 3, 128, 16), (2, 2, 48, 16)])
+def test_paged_attention_portions_and_window(ops_for, dtype, n_heads, n_kv, hd, page_size):
+    """Rows of prompt portions that start anywhere, beside single rows; and a window that ends mid-page."""
+    ops = ops_for(dtype)
+    group = n_heads // n_kv
+    kv_lens = [150, 77, 200, 5]
+    plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page_size, dtype, seed=30)
+    # request 0: rows at positions 100..149; request 1: its last row; request 2: positions 0..199; request 3: 3..4
+    segs = [(0, 100, 50), (1, 76, 1), (2, 0, 200), (3, 3, 2)]
+    positions, row_seq, seq_rows = [], [], []
+    for s, p0, n in segs:
+        seq_rows.append((len(positions), p0, n))
+        positions += list(range(p0, p0 + n)); row_seq += [s] * n
+    R = len(positions)
+    q = rnd((R, n_heads * hd), dtype, 31)
+    batch = SimpleNamespace(positions=torch.tensor(positions, dtype=torch.int32).cuda(),
+                            row_seq=torch.tensor(row_seq, dtype=torch.int32).cuda(),
+                            block_tables={"g": tables.cuda()}, max_kv_len=max(kv_lens), extras={},
+                            n_rows=R, max_seq_rows=200, seq_rows=seq_rows)
+    t = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    for window in (0, 37):
+        got = ops.paged_attention(q.cuda(), plane.cuda(), batch, "g", n_heads, n_kv, hd, window=window).cpu()
+        for r in range(0, R, 7):
+            want = dense_reference(q[r].view(n_heads, hd), ks[row_seq[r]], vs[row_seq[r]], group, positions[r], window)
+            torch.testing.assert_close(got[r].view(n_heads, hd).double(), want, **t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_one_far_key_among_hundreds(ops_for, dtype):
+    """One key far back is made to dominate: a kernel that skips a page or a split would miss it."""
+    ops = ops_for(dtype)
+    n_heads, n_kv, hd, page_size, L = 4, 2, 64, 16, 900
+    plane, tables, ks, vs = make_paged([L], n_kv, hd, page_size, dtype, seed=40)
+    q = rnd((1, n_heads * hd), dtype, 41)
+    for far in (0, 15, 16, 511, 512, 899):
+        k, v = ks[0].clone(), vs[0].clone()
+        k[far] = (q.view(n_heads, hd)[::2] * 4).to(dtype)            # aligned with the query of each kv head's first q head
+        page = tables[0, far // page_size].item()
+        pl = plane.clone()
+        pl[page, 0, :, far % page_size] = k[far]
+        batch = SimpleNamespace(positions=torch.tensor([L - 1], dtype=torch.int32).cuda(),
+                                row_seq=torch.zeros(1, dtype=torch.int32).cuda(), block_tables={"g": tables.cuda()},
+                                max_kv_len=L, extras={}, n_rows=1, max_seq_rows=1, seq_rows=[(0, L - 1, 1)])
+        got = ops.paged_attention(q.cuda(), pl.cuda(), batch, "g", n_heads, n_kv, hd).cpu().view(n_heads, hd)
+        want = dense_reference(q.view(n_heads, hd), k, v, 2, L - 1)
+        t = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(got.double(), want, **t)
+        # the dominated heads return (almost) the far value itself
+        assert (got[0].double() - v[far, 0].double()).abs().max() < 0.05
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,page_size,interleaved", [(8, 2, 8, 16, False), (3, 1, 32, 8, False),
+                                                                    (12, 3, 128, 16, False), (4, 2, 48, 4, True)])
+def test_rope_and_cache_write(ops_for, dtype, n_heads, n_kv, hd, page_size, interleaved):
+    ops, ref = ops_for(dtype), TorchOps(dtype=dtype)
+    n, n_pages, max_ctx = 23, 9, 300
+    j = torch.arange(hd // 2)
+    theta = 1.0 / torch.pow(torch.tensor(500000.0), (2 * j.float()) / hd)
+    ang = torch.outer(torch.arange(max_ctx).float(), theta)
+    table = torch.stack((torch.cos(ang), torch.sin(ang)), -1).contiguous()
+    qkv = rnd((n, (n_heads + 2 * n_kv) * hd), dtype, 50)
+    positions = torch.tensor(random.Random(51).sample(range(max_ctx), n), dtype=torch.int32)
+    slots = torch.tensor(random.Random(52).sample(range(n_pages * page_size), n), dtype=torch.int32)
+    plane0 = rnd((n_pages, 2, n_kv, page_size, hd), dtype, 53)
+    a, pa = qkv.clone().cuda(), plane0.clone().cuda()
+    ops.rope_write_kv(a, positions.cuda(), slots.cuda(), table.cuda(), pa, n_heads, n_kv, hd, page_size, interleaved)
+    b, pb = qkv.clone(), plane0.clone()
+    ref.rope_write_kv(b, positions, slots, table, pb, n_heads, n_kv, hd, page_size, interleaved)
+    t = tol(dtype)
+    torch.testing.assert_close(a.cpu()[:, :n_heads * hd].float(), b[:, :n_heads * hd].float(), **t)
+    torch.testing.assert_close(pa.cpu().float(), pb.float(), **t)
+    # position 0 is the identity; a unit vector at position 1 lands on cos 1 and sin 1 of its pair
+    one = torch.zeros(2, (n_heads + 2 * n_kv) * hd, dtype=dtype)
+    one[:, 0] = 1
+    g = one.clone().cuda()
+    ops.rope_write_kv(g, torch.tensor([0, 1], dtype=torch.int32).cuda(), slots[:2].cuda(), table.cuda(), pa, n_heads,
+                      n_kv, hd, page_size, interleaved)
+    g = g.cpu().float()
+    assert torch.equal(g[0], one[0].float())
+    partner = 1 if interleaved else hd // 2
+    assert abs(g[1, 0] - math.cos(1)) < 1e-2 and abs(g[1, partner] - math.sin(1)) < 1e-2
+    # reading without writing leaves the cache alone
+    before = pa.clone()
+    ops.rope_write_kv(qkv.clone().cuda(), positions.cuda(), slots.cuda(), table.cuda(), pa, n_heads, n_kv, hd,
+                      page_size, interleaved, write_cache=False)
+    assert torch.equal(before, pa)
+
+
+@pytest.mark.parametrize("V", [6, 100, 1000, 48000])
+def test_sampling(ops_for, V):
+    ops, ref = ops_for(torch.float32), TorchOps()
+    n = 8
+    logits = rnd((n, V), torch.float32, 60, 3.0)
+    temperature = torch.tensor([0.0, 1.0, 0.8, 1.0, 0.9, 1.3, 1.0, 0.7])
+    top_k = torch.tensor([0, 1, 0, 3, 50, 0, 0, 5], dtype=torch.int32)
+    top_p = torch.tensor([0.0, 0.0, 0.0, 0.9, 0.95, 0.5, 0.0, 0.3])
+    pen = torch.tensor([1.0, 1.0, 1.0, 1.0, 1.1, 1.0, 1.3, 2.0])
+    ctx = [torch.tensor(random.Random(61 + i).choices(range(V), k=7), dtype=torch.int32) for i in range(n)]
+    off = torch.tensor([0] + list(torch.tensor([len(c) for c in ctx]).cumsum(0)), dtype=torch.int32)
+    ctx_t = torch.cat(ctx)
+    for trial in range(6):
+        u = torch.rand(n, generator=torch.Generator().manual_seed(70 + trial))
+        got = ops.sample(logits.cuda(), temperature.cuda(), top_k.cuda(), top_p.cuda(), pen.cuda(), u.cuda(),
+                         ctx_t.cuda(), off.cuda()).cpu()
+        want = ref.sample(logits, temperature, top_k, top_p, pen, u, ctx_t, off)
+        assert got.tolist() == want.tolist(), (trial, got.tolist(), want.tolist())
+    assert ops.argmax(logits.cuda()).cpu().tolist() == logits.argmax(-1).tolist()
+
+
+def test_sampling_reference_vectors(ops_for):
+    """The reference's own vector (test_server.py:120-122): a repetition penalty pushes token 5 below token 7."""
+    ops = ops_for(torch.float32)
+    lg = torch.zeros(1, 100); lg[0, 5] = 5.0; lg[0, 7] = 4.9
+    one = lambda v, dt=torch.float32: torch.tensor([v], dtype=dt).cuda()
+    args = (one(1.0), one(1, torch.int32), one(0.0))
+    assert ops.sample(lg.cuda(), *args, one(1.0), one(0.5)).item() == 5
+    assert ops.sample(lg.cuda(), *args, one(2.0), one(0.5), one(5, torch.int32), torch.tensor([0, 1], dtype=torch.int32).cuda()).item() == 7

@@ -1,0 +1,209 @@
+"""Continuous batching above the step function: admit, cut prompts into portions, decode, finish, free.
+
+Follows the reference's scheduler (server.py:101-292, 475-479) where it has a rule, and adds what it lacks: a
+token budget per step, under which prompts are fed in portions beside the decode tokens of other requests,
+all in one batch (the reference prefills whole prompts in a launch of their own, server.py:279-284).
+
+Admission (server.py:138-168): a queued request joins while a batch slot is free and the page plan allows.
+plan "final" admits while every running request still fits at its full length (prompt + max_new_tokens), so
+nothing is ever preempted; plan "cur" admits on what requests hold now, against a running budget, and lets
+them outgrow the pool.
+
+When pages run out (server.py:187-193, 261-269): before a step runs, while the step's new pages exceed the
+free ones, the newest running request is taken out, its pages and state slot are given back, and it goes to
+the front of the queue; later it is fed again from its prompt plus what it had generated, and its random
+stream goes on where it was. A lone request that does not fit is an error.
+
+Finishing (server.py:242-252): the end-of-sequence token, max_new_tokens, or the model's context.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, List, Optional, Sequence
+
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+
+
+class Request:
+    _next_id = 0
+
+    def __init__(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None, **kw):
+        if len(prompt_ids) == 0:
+            raise ValueError("a request needs at least one prompt token")
+        self.id = Request._next_id
+        Request._next_id += 1
+        self.ids: List[int] = [int(t) for t in prompt_ids]      # committed tokens: prompt + generated
+        self.prompt_len = len(self.ids)
+        self.params = params or SamplingParams(**kw)
+        self.fed = 0            # positions whose keys and values are in the cache
+        self.done = False
+        self.preempted = 0
+
+    def out_ids(self) -> List[int]:
+        return self.ids[self.prompt_len:]
+
+
+@dataclass
+class StepPlan:
+    """What one step will run: (request, first position, number of tokens, sample afterwards?)."""
+    items: List[tuple] = field(default_factory=list)
+
+    @property
+    def n_tokens(self) -> int:
+        return sum(n for _, _, n, _ in self.items)
+
+
+def pages_for(n_tokens: int, page_size: int) -> int:
+    return -(-n_tokens // page_size)
+
+
+class Scheduler:
+    def __init__(self, engine, max_batch: int = 8, token_budget: int = 2048, plan: str = "final",
+                 max_context: Optional[int] = None):
+        if plan not in ("final", "cur"):
+            raise ValueError(f"plan {plan!r}: use 'final' or 'cur'")
+        if max_batch < 1:
+            raise ValueError(f"max_batch must be at least 1, got {max_batch}")
+        if token_budget < max_batch:
+            raise ValueError(f"token_budget {token_budget} must give every one of {max_batch} requests a token")
+        self.engine = engine
+        self.max_batch = min(max_batch, engine.cache.max_requests)
+        self.token_budget = token_budget
+        self.plan = plan
+        self.max_context = min(max_context or engine.spec.max_context, engine.spec.max_context)
+        self.eos = engine.spec.eos_token_id
+        self.page_size = engine.page_size
+        self.sampler = Sampler(engine.ops)
+        self.queue: Deque[Request] = deque()
+        self.active: List[Request] = []
+        self.finished: List[Request] = []
+        self.preempts = 0
+        self.replays = 0            # preempted after work was done: that work is done again
+        self.peak_running = 0
+        self.steps = 0
+        self.tokens_run = 0
+
+    # ---- queueing and admission ----------------------------------------------------------------------
+    def submit(self, req: Request) -> None:
+        if req.prompt_len >= self.max_context:
+            raise ValueError(f"a prompt of {req.prompt_len} tokens leaves no room in a context of {self.max_context}")
+        self.queue.append(req)
+
+    def _held(self, r: Request) -> int:
+        return pages_for(r.fed, self.page_size) if r.fed else 0
+
+    def _grow_pages(self, r: Request, n_new: int) -> int:
+        """Pages r must take to be fed n_new more tokens."""
+        return pages_for(r.fed + n_new, self.page_size) - self._held(r)
+
+    def _final_pages(self, r: Request) -> int:
+        """Pages r holds once it has generated all it may (the last token is sampled, never fed)."""
+        return pages_for(min(r.prompt_len + r.params.max_new_tokens - 1, self.max_context), self.page_size)
+
+    def admit(self) -> None:
+        total = self.engine.total_pages()
+        # pages are only taken when a request runs, so the free count does not move while admitting: keep a
+        # budget instead (the reference's fix, server.py:143-147)
+        budget = self.engine.free_pages() - sum(self._grow_pages(r, 1) for r in self.active)
+        while self.queue and len(self.active) < self.max_batch:
+            q = self.queue[0]
+            need_now = pages_for(len(q.ids), self.page_size)
+            if self.plan == "final":
+                projected = sum(self._final_pages(r) for r in self.active) + self._final_pages(q)
+                if projected > total and self.active:
+                    break
+            elif need_now > budget and self.active:
+                break
+            budget -= need_now
+            self.queue.popleft()
+            q.fed = 0
+            self.active.append(q)
+
+    # ---- one step ------------------------------------------------------------------------------------
+    def plan_step(self) -> StepPlan:
+        """Decode tokens first, then prompt portions in admission order, under the token budget."""
+        plan = StepPlan()
+        left = self.token_budget
+        for r in self.active:
+            if len(r.ids) - r.fed == 1 and r.fed >= r.prompt_len:
+                plan.items.append((r, r.fed, 1, True))
+                left -= 1
+        for r in self.active:
+            pending = len(r.ids) - r.fed
+            if pending >= 1 and not (pending == 1 and r.fed >= r.prompt_len):
+                if left <= 0:
+                    continue
+                n = min(pending, left)
+                plan.items.append((r, r.fed, n, n == pending))
+                left -= n
+        return plan
+
+    def preempt(self) -> None:
+        r = self.active.pop()
+        self.preempts += 1
+        if r.fed > 0:
+            self.replays += 1
+        if r.id in self.engine.requests:
+            self.engine.close(r.id)
+        r.fed = 0
+        r.preempted += 1
+        self.queue.appendleft(r)
+
+    def step(self) -> None:
+        if not self.active:
+            return
+        while True:
+            plan = self.plan_step()
+            need = sum(self._grow_pages(r, n) for r, _, n, _ in plan.items)
+            if need <= self.engine.free_pages():
+                break
+            if len(self.active) == 1:
+                r = self.active[0]
+                raise RuntimeError("kv pool too small for a single request: "
+                                   f"{len(r.ids)} tokens need {pages_for(len(r.ids), self.page_size)} pages of "
+                                   f"{self.page_size}, the pool has {self.engine.total_pages()}")
+            self.preempt()
+        self.peak_running = max(self.peak_running, len(self.active))
+        if not plan.items:
+            return
+        entries = []
+        for r, start, n, sample in plan.items:
+            entries.append((r.id, r.ids[start:start + n], [n - 1] if sample else []))
+        out = self.engine.step(entries)
+        self.steps += 1
+        self.tokens_run += plan.n_tokens
+        sampled = [r for r, _, _, s in plan.items if s]
+        for r, _, n, _ in plan.items:
+            r.fed += n
+        if sampled:
+            toks = self.sampler.sample(out.logits, [r.params for r in sampled],
+                                       [len(r.out_ids()) for r in sampled], [r.ids for r in sampled])
+            for r, t in zip(sampled, toks):
+                r.ids.append(int(t))
+                self.finish_check(r)
+        for r in self.active:
+            if r.done:
+                self.engine.close(r.id)
+                self.finished.append(r)
+        self.active = [r for r in self.active if not r.done]
+
+    def finish_check(self, r: Request) -> None:
+        out = r.out_ids()
+        if self.eos >= 0 and not r.params.ignore_eos and self.eos in out:
+            r.ids = r.ids[:r.prompt_len + out.index(self.eos) + 1]
+            r.done = True
+        if len(r.out_ids()) >= r.params.max_new_tokens:
+            r.ids = r.ids[:r.prompt_len + r.params.max_new_tokens]
+            r.done = True
+        if len(r.ids) >= self.max_context:
+            r.done = True
+
+    def run(self) -> List[Request]:
+        while self.queue or self.active:
+            self.admit()
+            if not self.active:
+                raise RuntimeError("nothing can be admitted: is max_batch 0 or the pool empty?")
+            self.step()
+        return self.finished

@@ -127,7 +127,7 @@ def make_paged(kv_lens, n_kv, hd, page_size, dtype, seed, shuffle=True):
         pages = [ids.pop() for _ in range(-(-L // page_size))]
         for j in range(L):
             plane[pages[j // page_size], 0, :, j % page_size] = k[j]
-            plane[pages[j // page_size], 1, :, j % page_size] = v[j]
+            plane[pages[j // page_size], 1].view(n_kv, hd, page_size)[:, :, j % page_size] = v[j]     # values lie transposed
         tables.append(pages + [0] * (width - len(pages)))
         ks.append(k); vs.append(v)
     return plane, torch.tensor(tables, dtype=torch.int32), ks, vs

@@ -89,8 +89,11 @@ class TorchOps:
         if write_cache:
             slots = write_slots.long()
             page, off = slots // page_size, slots % page_size
+            # a page holds keys as [kv head][slot][head_dim] and values transposed, [kv head][head_dim][slot]
             plane[page, 0, :, off] = x[:, n_heads:n_heads + n_kv_heads]
-            plane[page, 1, :, off] = x[:, n_heads + n_kv_heads:]
+            vt = plane[:, 1].reshape(plane.shape[0], n_kv_heads, head_dim, page_size)
+            vt[page, :, :, off] = x[:, n_heads + n_kv_heads:]
+            plane[:, 1] = vt.reshape(plane.shape[0], n_kv_heads, page_size, head_dim)
 
     # ---- attention over the paged cache -----------------------------------------------------------------
     def paged_attention(self, q, plane, batch, group, n_heads, n_kv_heads, head_dim, window=0, scale=None):
@@ -108,7 +111,8 @@ class TorchOps:
             js = torch.arange(first, p + 1)
             pages = tables[seq[r]].long()[js // page_size]
             k = plane[pages, 0, :, js % page_size].float()       # [keys, kvh, hd]
-            v = plane[pages, 1, :, js % page_size].float()
+            vt = plane[:, 1].reshape(plane.shape[0], n_kv_heads, head_dim, page_size)
+            v = vt[pages, :, :, js % page_size].float()
             qr = q[r].float().view(n_heads, head_dim)
             for h in range(n_heads):
                 s = (k[:, h // g] @ qr[h]) * scale

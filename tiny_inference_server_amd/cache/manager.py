@@ -92,8 +92,10 @@ class PageGroup:
         self.released: Dict[int, int] = {}               # slot -> number of leading pages already given back
         self.storage = None
         if allocate:
-            # [plane][page][key or value][kv head][slot in page][head size]
-            self.storage = torch.empty((len(spec.keys), n_pages, 2, spec.n_kv_heads, page_size, spec.head_dim),
+            # [plane][page][key or value][kv head][slot in page][head size]; within a page and head the values
+            # lie transposed, [head size][slot]. Zeroed once: kernels that multiply masked slots by an exact 0
+            # need every value ever found in the pool to be finite (the reference zeroes too: block_table.py:40)
+            self.storage = torch.zeros((len(spec.keys), n_pages, 2, spec.n_kv_heads, page_size, spec.head_dim),
                                        dtype=dtype, device=device)
 
     def plane(self, key: str):

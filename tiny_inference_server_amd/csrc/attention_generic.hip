@@ -5,6 +5,7 @@
 // table. Query head h reads key/value head h / group_size (reference paged_attention_kernels.py:49).
 // Scores, maximum, sum and the output accumulate in 32-bit (reference paged_attention_kernels.py:86-108);
 // masked keys are never read, so what a reused page still holds cannot reach the result.
+// A page holds a head's keys as [slot][head_dim] and its values as [head_dim][slot].
 // Keys are walked in chunks of a fixed size with a running maximum, so the order of every sum depends on
 // the row's own length only, not on what else is in the batch.
 #include "common.h"
@@ -73,8 +74,8 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     if (pv_thread) {
       for (int i = g; i < n; i += groups) {
         const int j = c0 + i;
-        const T* vp = plane + (long)bt[j / page_size] * page_stride + v_off + (long)(j % page_size) * HD;
-        acc += sc[i] * to_f(vp[d]);
+        const T* vp = plane + (long)bt[j / page_size] * page_stride + v_off + (j % page_size);
+        acc += sc[i] * to_f(vp[(long)d * page_size]);  // values lie transposed: [head_dim][slot]
       }
     }
     __syncthreads();  // sc[] is rewritten by the next chunk

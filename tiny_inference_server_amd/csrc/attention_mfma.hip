@@ -1,0 +1,285 @@
+// Attention over paged keys and values on the matrix cores (bfloat16, gfx950), for decode rows and for
+// portions of prompts alike. Compiled for one head size: -DTIS_HD=<multiple of 16, at most 256>.
+//
+// One wavefront owns an *item*: up to 16*NB query columns that share a request and a key/value head, a
+// column being (row, query head): n_rows consecutive positions of the request times the group's query heads.
+// A decode row is an item of one row; all query heads of its group share one pass over the keys, so keys
+// and values are read once per group, not once per query head. A long key range is cut into splits that
+// different wavefronts take; a second kernel merges their partial results.
+//
+// Per step of 32 keys (two tiles of 16, each inside one page; page sizes are multiples of 16):
+//   S^T[key, col] = K[key, :] . Q[col, :]      v_mfma_f32_16x16x32_bf16, A = keys straight from the page
+//                                              ([slot][head_dim]: 16 bytes per lane), B = queries in registers
+//   mask by select (key <= the column's position, key inside its window), running maximum and sum per column
+//   in 32-bit, base-2 exponentials with log2(e)/sqrt(head_dim) folded into the scale
+//   O^T[d, col] += V^T[d, key] . P^T[key, col] A = values straight from the page, which holds them transposed
+//                                              ([head_dim][slot]: 8 bytes per lane and tile), B = P rounded to
+//                                              bfloat16 (as the reference does before P.V:
+//                                              paged_attention_kernels.py:108), exactly as S^T left it in registers
+// Both products put the column on the lane, so the softmax statistics never cross lanes except for the
+// reduction over the four key groups, and no LDS is used. Masked keys are read but multiplied by an exact 0:
+// every value ever found in the pool must be finite, which the pool's one-time zeroing ensures.
+#include "common.h"
+
+#ifndef TIS_HD
+#error "compile with -DTIS_HD=<head size>"
+#endif
+static_assert(TIS_HD % 16 == 0 && TIS_HD >= 16 && TIS_HD <= 256, "head size must be a multiple of 16, at most 256");
+
+TIS_DEFINE_LAST_ERROR(tis_attention_mfma)
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+static constexpr int HD = TIS_HD;
+static constexpr int DC = (HD + 31) / 32;   // 32-wide chunks of the head for Q.K
+static constexpr int DB = HD / 16;          // 16-wide blocks of the head for P.V
+
+__device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x4 load4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
+
+template <int NB>
+__global__ __launch_bounds__(64) void attention_mfma_kernel(
+    const bf16* __restrict__ q, long q_ld, const bf16* __restrict__ plane, const int* __restrict__ block_tables,
+    int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ items,
+    bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
+    int n_kv_heads, int n_heads, int page_size, int window, float scale_log2, int n_splits) {
+  const int item = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  const int lane = threadIdx.x, c16 = lane & 15, g = lane >> 4;
+  const int row0 = items[item].x, n_rows = items[item].y;
+  const int* bt = block_tables + (long)row_seq[row0] * bt_ld;
+  const int p_first = positions[row0];
+  const int p_last = p_first + n_rows - 1;
+
+  // the lane's column in each block
+  int col_row[NB], col_head[NB], col_pos[NB], col_lo[NB];
+  bool col_ok[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int c = nb * 16 + c16;
+    const int ro = c / group_size;
+    col_ok[nb] = ro < n_rows;
+    col_row[nb] = row0 + (col_ok[nb] ? ro : 0);
+    col_head[nb] = kvh * group_size + c % group_size;
+    col_pos[nb] = col_ok[nb] ? p_first + ro : -1;
+    col_lo[nb] = (window > 0 && col_pos[nb] - window + 1 > 0) ? col_pos[nb] - window + 1 : 0;
+  }
+
+  // queries: the B operand of S^T, kept in registers for the whole key range
+  bf16x8 qb[NB][DC];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) {
+      const int d = dc * 32 + g * 8;
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (col_ok[nb] && d < HD) v = load8(q + (long)col_row[nb] * q_ld + (long)col_head[nb] * HD + d);
+      qb[nb][dc] = v;
+    }
+
+  // this wave's share of the item's keys, in steps of 32 from a multiple of 32
+  int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+  k_lo &= ~31;
+  const int k_hi = p_last + 1;
+  const int n_steps = (k_hi - k_lo + 31) / 32;
+  const int per_split = (n_steps + n_splits - 1) / n_splits;
+  const int s_begin = split * per_split;
+  const int s_end = min(n_steps, s_begin + per_split);
+
+  const long page_stride = 2L * n_kv_heads * page_size * HD;
+  const long k_head = (long)kvh * page_size * HD;
+  const long v_head = ((long)n_kv_heads + kvh) * page_size * HD;
+
+  f32x4 o[NB][DB];
+  float m[NB], l[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    m[nb] = -INFINITY;
+    l[nb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) o[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int s = s_begin; s < s_end; ++s) {
+    const int kb = k_lo + s * 32;
+    // page and first slot of the two 16-key tiles; a tile past the item's last key is skipped
+    bool tile_ok[2];
+    const bf16* kp[2];
+    const bf16* vp[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key0 = kb + t * 16;
+      tile_ok[t] = key0 < k_hi;
+      const long page = tile_ok[t] ? bt[key0 / page_size] : 0;
+      const int slot0 = key0 % page_size;
+      kp[t] = plane + page * page_stride + k_head + (long)(slot0 + c16) * HD + g * 8;
+      vp[t] = plane + page * page_stride + v_head + (long)c16 * page_size + slot0 + g * 4;
+    }
+    // S^T = K . Q^T
+    f32x4 st[2][NB];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) st[t][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      if (tile_ok[t]) {
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+          bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0};
+          if (dc * 32 + g * 8 < HD) ka = load8(kp[t] + dc * 32);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+            st[t][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[nb][dc], st[t][nb], 0, 0, 0);
+        }
+      }
+    }
+    // mask, running maximum and sum per column, P in bfloat16 as the B operand of the second product
+    bf16x8 pb[NB];
+    float alpha[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float sv[8];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + t * 16 + g * 4 + i;
+          const bool ok = tile_ok[t] && key <= col_pos[nb] && key >= col_lo[nb];
+          const float v = ok ? st[t][nb][i] * scale_log2 : -INFINITY;
+          sv[t * 4 + i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m[nb], tmax);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a column with no key yet: everything stays 0
+      alpha[nb] = exp2f(m[nb] - m_use);
+      float psum = 0.f;
+      bf16x8 pv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = exp2f(sv[e] - m_use);
+        psum += p;
+        pv[e] = static_cast<__bf16>(p);
+      }
+      pb[nb] = pv;
+      l[nb] = l[nb] * alpha[nb] + psum;      // the lane's share; the four key groups are added at the end
+      m[nb] = m_new;
+    }
+    // O^T = O^T * alpha + V^T . P^T
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      bf16x8 va;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        bf16x4 h = {0, 0, 0, 0};
+        if (tile_ok[t]) h = load4(vp[t] + (long)db * 16 * page_size);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) va[t * 4 + e] = h[e];
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        f32x4 acc = o[nb][db];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] *= alpha[nb];
+        o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[nb], acc, 0, 0, 0);
+      }
+    }
+  }
+
+  // the lane holds, for its column, the outputs d = db*16 + g*4 + {0..3}
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    float lt = l[nb];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    if (!col_ok[nb]) continue;
+    if (n_splits == 1) {
+      const float inv = 1.f / lt;
+      bf16* dst = out + (long)col_row[nb] * out_ld + (long)col_head[nb] * HD + g * 4;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        bf16x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = static_cast<__bf16>(o[nb][db][i] * inv);
+        *reinterpret_cast<bf16x4*>(dst + db * 16) = w;
+      }
+    } else {
+      const long slot = ((long)col_row[nb] * n_heads + col_head[nb]) * n_splits + split;
+      float* dst = part_o + slot * HD + g * 4;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + db * 16) = o[nb][db];
+      if (g == 0) part_ml[slot] = make_float2(m[nb], lt);
+    }
+  }
+}
+
+// out[row, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s      (reference paged_attention_kernels.py:121-204)
+__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ part_o,
+                                                             const float2* __restrict__ part_ml,
+                                                             bf16* __restrict__ out, long out_ld, int n_heads,
+                                                             int n_splits) {
+  const long row = blockIdx.x;
+  const int head = blockIdx.y;
+  const long base = (row * n_heads + head) * n_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[base + s].x);
+  float L = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float2 ml = part_ml[base + s];
+    if (ml.x > -INFINITY) L += exp2f(ml.x - M) * ml.y;
+  }
+  for (int d = threadIdx.x; d < HD; d += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float mx = part_ml[base + s].x;
+      if (mx > -INFINITY) acc += exp2f(mx - M) * part_o[(base + s) * HD + d];
+    }
+    out[row * out_ld + (long)head * HD + d] = static_cast<__bf16>(acc / L);
+  }
+}
+
+TIS_EXPORT int tis_attention_mfma_head_dim() { return HD; }
+
+// items: (first row, rows) pairs; the rows of an item are consecutive positions of one request and
+// rows * group_size <= 16 * nb. part_o / part_ml: workspace for n_splits > 1, [rows][heads][splits][HD] floats and
+// [rows][heads][splits] float pairs.
+TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
+                                  const int* row_seq, const int* positions, const int* items, int n_items, int nb,
+                                  void* out, long out_ld, float* part_o, float* part_ml, int rows, int n_heads,
+                                  int n_kv_heads, int head_dim, int page_size, int window, float scale, int n_splits,
+                                  hipStream_t stream) {
+  if (n_items == 0 || rows == 0) return 0;
+  if (head_dim != HD) return tis_fail("attention_mfma: built for head size %d, called with %d", HD, head_dim);
+  if (n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads)
+    return tis_fail("attention_mfma: %d query heads over %d key/value heads", n_heads, n_kv_heads);
+  const int group = n_heads / n_kv_heads;
+  if (nb != 1 && nb != 2 && nb != 4) return tis_fail("attention_mfma: %d column blocks; 1, 2 or 4 are built", nb);
+  if (group > 16 * nb) return tis_fail("attention_mfma: a group of %d query heads does not fit %d columns", group, 16 * nb);
+  if (page_size < 16 || page_size % 16) return tis_fail("attention_mfma: page size %d is no multiple of 16", page_size);
+  if (n_splits < 1 || n_splits > 65535 || n_kv_heads > 65535) return tis_fail("attention_mfma: bad grid %d x %d", n_kv_heads, n_splits);
+  if (n_splits > 1 && (!part_o || !part_ml)) return tis_fail("attention_mfma: %d splits need a workspace", n_splits);
+  if ((q_ld % 8) || (out_ld % 4) || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)plane % 16))
+    return tis_fail("attention_mfma: q, out and the cache plane must be 16-byte aligned with row strides in steps of 8");
+  dim3 grid(n_items, n_kv_heads, n_splits);
+  const float scale_log2 = scale * 1.4426950408889634f;
+#define LAUNCH(NBV)                                                                                              \
+  attention_mfma_kernel<NBV><<<grid, 64, 0, stream>>>(                                                           \
+      (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)items,     \
+      (bf16*)out, out_ld, part_o, (float2*)part_ml, group, n_kv_heads, n_heads, page_size, window, scale_log2,   \
+      n_splits)
+  if (nb == 1) LAUNCH(1);
+  else if (nb == 2) LAUNCH(2);
+  else LAUNCH(4);
+#undef LAUNCH
+  int rc = tis_launch_status("attention_mfma");
+  if (rc) return rc;
+  if (n_splits > 1) {
+    dim3 mgrid(rows, n_heads);
+    attention_merge_kernel<<<mgrid, 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld, n_heads,
+                                                     n_splits);
+    rc = tis_launch_status("attention_merge");
+  }
+  return rc;
+}

@@ -5,7 +5,8 @@
 // (cos, sin) per position and pair. Pairs are (j, j + head_dim/2) in the "half" pairing (reference
 // main_models_new.py:71-80) or (2j, 2j+1) in the "interleaved" pairing; a null table means no rotation.
 //
-// One cache plane is laid out [page][key or value][kv head][slot in page][head_dim].
+// One cache plane is laid out [page][key or value][kv head][...]: a head's keys of a page as [slot][head_dim],
+// its values transposed as [head_dim][slot], which is how the matrix-core attention kernel wants to load them.
 #include "common.h"
 
 TIS_DEFINE_LAST_ERROR(tis_rope_cache)
@@ -31,10 +32,16 @@ __global__ __launch_bounds__(64) void rope_write_kv_kernel(T* __restrict__ qkv, 
       const int slot = write_slots[r];
       const int page = slot / page_size, off = slot % page_size;
       const int kvh = is_v ? hh - n_heads - n_kv_heads : hh - n_heads;
-      dst = plane + ((((long)page * 2 + (is_v ? 1 : 0)) * n_kv_heads + kvh) * page_size + off) * head_dim;
+      T* head = plane + (((long)page * 2 + (is_v ? 1 : 0)) * n_kv_heads + kvh) * page_size * head_dim;
+      if (is_v) {  // values: [head_dim][slot]
+        for (int i = threadIdx.x; i < head_dim; i += blockDim.x) head[(long)i * page_size + off] = row[i];
+        return;
+      }
+      dst = head + (long)off * head_dim;
     }
   }
-  if (is_v || table == nullptr) {
+  if (is_v) return;
+  if (table == nullptr) {
     if (dst != row)
       for (int i = threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = row[i];
     return;

@@ -93,7 +93,7 @@ class _Packer:
 
 
 def build_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: Sequence[bool], cache, device,
-                     max_context: int) -> StepBatch:
+                     max_context: int, plan_rows=None) -> StepBatch:
     """Row arrays for every stage of one step. `cache` is the CacheManager that already covers the new positions."""
     n_seqs = len(entries)
     pk = _Packer()
@@ -158,8 +158,9 @@ def build_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: 
                 ok = p >= p0 and n > 0
                 want.append(first_row + (p - p0) if ok else -1)
                 valid.append(ok)
+        extra = plan_rows(seq_rows, pk.add) if plan_rows is not None else {}
         plans.append(dict(
-            lag=lag, n_rows=len(tokens), tokens=pk.add(tokens), positions=pk.add(positions),
+            extra=extra, lag=lag, n_rows=len(tokens), tokens=pk.add(tokens), positions=pk.add(positions),
             row_seq=pk.add(row_seq), cu=pk.add(cu), ws=ws,
             source=pk.add(source) if has_source[j] else None,
             keep_src=pk.add(keep_src) if has_source[j] else None,
@@ -181,5 +182,6 @@ def build_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: 
             keep_source=dev[pl["keep_src"]] if pl["keep_src"] is not None else None,
             keep_slot=dev[pl["keep_slot"]] if pl["keep_slot"] is not None else None,
             keep_count=pl["keep_count"], want_index=dev[pl["want"]], want_valid=pl["valid"],
-            max_kv_len=pl["max_kv"], max_seq_rows=pl["max_rows"], seq_rows=pl["seq_rows"]))
+            max_kv_len=pl["max_kv"], max_seq_rows=pl["max_rows"], seq_rows=pl["seq_rows"],
+            extras={k: (dev[v[0]],) + tuple(v[1:]) for k, v in pl["extra"].items()}))
     return StepBatch(list(entries), stages, sum(len(e.want) for e in entries))

@@ -131,8 +131,7 @@ class Engine:
             self.cache.grow(slot, fed + len(toks))
             batch_entries.append(Entry(slot, fed, list(toks), list(want)))
         step = build_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache, self.device,
-                                self.spec.max_context)
-        self.plan(step)
+                                self.spec.max_context, getattr(self.ops, "plan_rows", None))
         outs = self.model.forward(step, self.cache)
         n = step.n_wanted
         vocab = self.spec.vocab_size
@@ -158,9 +157,3 @@ class Engine:
             self.requests[rid] = (slot, fed + len(toks))
             self.cache.release_behind(slot, fed + len(toks), self.model.max_lag)
         return StepOutput(logits, head_logits, head_valid)
-
-    def plan(self, step) -> None:
-        """Host-side planning that the kernels of this ops object want for a step (none for the plain kernels)."""
-        planner = getattr(self.ops, "plan_step", None)
-        if planner is not None:
-            planner(step, self.cache)

@@ -50,7 +50,16 @@ class BuildError(RuntimeError):
 
 
 def available_sources() -> List[str]:
-    return [n for n, f in SOURCES.items() if os.path.isfile(os.path.join(CSRC, f))]
+    """Every library that build() makes by default, variants spelled out."""
+    out = []
+    for n, f in SOURCES.items():
+        if not os.path.isfile(os.path.join(CSRC, f)):
+            continue
+        if n in VARIANTS:
+            out.extend(f"{n}@{v}" for v in VARIANTS[n][1])
+        else:
+            out.append(n)
+    return out
 
 
 def _hipcc() -> str:
@@ -60,12 +69,31 @@ def _hipcc() -> str:
     raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin): the HIP kernels cannot be built")
 
 
+# libraries compiled once per value of a macro: name -> (macro, values that build() makes without being asked)
+VARIANTS: Dict[str, tuple] = {
+    "attention_mfma": ("TIS_HD", (32, 48, 64, 128, 256)),
+}
+
+
+def split_variant(name: str):
+    """'attention_mfma@128' -> ('attention_mfma', ['-DTIS_HD=128'])."""
+    if "@" not in name:
+        if name in VARIANTS:
+            raise BuildError(f"library {name!r} is built per {VARIANTS[name][0]}: ask for '{name}@<value>'")
+        return name, []
+    base, value = name.split("@", 1)
+    if base not in VARIANTS:
+        raise BuildError(f"library {base!r} has no variants")
+    return base, [f"-D{VARIANTS[base][0]}={int(value)}"]
+
+
 def _digest(name: str) -> str:
+    base, defines = split_variant(name)
     h = hashlib.sha1()
-    for f in [SOURCES[name]] + HEADERS:
+    for f in [SOURCES[base]] + HEADERS:
         with open(os.path.join(CSRC, f), "rb") as fh:
             h.update(fh.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + defines).encode())
     return h.hexdigest()[:12]
 
 
@@ -103,20 +131,21 @@ def library_file(name: str) -> Optional[str]:
 
 
 def _compile(name: str, out_dir: str) -> str:
-    src = os.path.join(CSRC, SOURCES[name])
+    base, defines = split_variant(name)
+    src = os.path.join(CSRC, SOURCES[base])
     out = os.path.join(out_dir, f"{name}.{_digest(name)}.so")
     tmp = f"{out}.tmp{os.getpid()}"
     env = dict(os.environ)
     if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
         env["HOME"] = out_dir   # the compiler may want a cache folder
-    cmd = [_hipcc()] + FLAGS + ["-I", CSRC, "-o", tmp, src]
+    cmd = [_hipcc()] + FLAGS + defines + ["-I", CSRC, "-o", tmp, src]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
     if proc.returncode != 0:
         try:
             os.remove(tmp)
         except OSError:
             pass
-        raise BuildError(f"hipcc failed on {SOURCES[name]}:\n{proc.stdout[-4000:]}")
+        raise BuildError(f"hipcc failed on {SOURCES[base]} ({name}):\n{proc.stdout[-4000:]}")
     os.replace(tmp, out)
     # older builds of the same library are of no further use
     for f in os.listdir(out_dir):
@@ -136,7 +165,7 @@ def build(names: Optional[Iterable[str]] = None, force: bool = False, log=None) 
     log = log or (lambda s: print(s, file=sys.stderr, flush=True))
     names = list(names) if names is not None else available_sources()
     for n in names:
-        if n not in SOURCES:
+        if split_variant(n)[0] not in SOURCES:
             raise BuildError(f"unknown kernel library {n!r}; known: {', '.join(SOURCES)}")
     result: Dict[str, str] = {}
     todo = []

@@ -74,15 +74,42 @@ _SIGNATURES = {
     }),
 }
 
+_SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
+    "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+})
+
 _libs = {}
 
 
 def library(name: str) -> _Lib:
+    """`name` may carry a variant: 'attention_mfma@128'."""
     lib = _libs.get(name)
     if lib is None:
-        prefix, sigs = _SIGNATURES[name]
+        prefix, sigs = _SIGNATURES[name.split("@")[0]]
         lib = _libs[name] = _Lib(name, prefix, sigs)
     return lib
+
+
+# wavefronts the attention launch aims for, so that short batches still spread over the chip
+_ATTN_TARGET_WAVES = 1024
+
+
+def attention_items(seq_rows, group_size: int):
+    """Work items of the matrix-core attention kernel for the rows of one stage.
+
+    seq_rows: (first row, first position, rows) per request. Returns (column blocks per item, [(first row, rows)]):
+    an item holds consecutive rows of one request, rows * group_size <= 16 * blocks.
+    """
+    single = all(n <= 1 for _, _, n in seq_rows)
+    nb = 1 if single else 2
+    while group_size > 16 * nb:
+        nb *= 2
+    per_item = max(1, (16 * nb) // group_size)
+    items = []
+    for first, _, n in seq_rows:
+        for r in range(0, n, per_item):
+            items.append((first + r, min(per_item, n - r)))
+    return nb, items
 
 
 def _rows_view(t: torch.Tensor, what: str):
@@ -108,6 +135,24 @@ class HipOps:
         self.attn_generic = library("attention_generic")
         self.gemm_plain = library("gemm_plain")
         self.sampling = library("sampling")
+        self._attn_groups = set()          # group sizes of the attention mixers built on these ops
+        self._attn_mfma = {}               # head size -> library
+        self._workspace = None
+
+    # ---- planning on the host --------------------------------------------------------------------------
+    def register_attention(self, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
+        """An attention mixer announces its shape, so that each step's work items are planned once, up front."""
+        self._attn_groups.add(n_heads // n_kv_heads)
+
+    def plan_rows(self, seq_rows, add):
+        """Called while a step's arrays are packed: returns {name: (packed array id, host values...)}."""
+        plans = {}
+        if self.dtype == torch.bfloat16:
+            for group in sorted(self._attn_groups):
+                nb, items = attention_items(seq_rows, group)
+                if nb <= 4 and items:
+                    plans[("attention_items", group)] = (add([v for it in items for v in it]), len(items), nb)
+        return plans
 
     # ---- helpers -------------------------------------------------------------------------------------
     def _stream(self):
@@ -307,6 +352,33 @@ class HipOps:
         if scale is None:
             scale = head_dim ** -0.5
         out = self.empty(n, n_heads * head_dim)
+        if n == 0:
+            return out
+        group = n_heads // n_kv_heads
+        if (self.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 16 == 0
+                and group <= 64 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0):
+            plan = batch.extras.get(("attention_items", group))
+            if plan is None:        # a caller that did not plan (a kernel test): plan now
+                nb, host_items = attention_items(batch.seq_rows, group)
+                items = torch.tensor(host_items, dtype=torch.int32).reshape(-1).to(self.device)
+                plan = (items, len(host_items), nb)
+            items, n_items, nb = plan
+            lib = self._attn_mfma.get(head_dim)
+            if lib is None:
+                lib = self._attn_mfma[head_dim] = library(f"attention_mfma@{head_dim}")
+            n_splits = max(1, min(-(-_ATTN_TARGET_WAVES // (n_items * n_kv_heads)), -(-batch.max_kv_len // 64)))
+            part_o = part_ml = None
+            if n_splits > 1:
+                need = n * n_heads * n_splits * (head_dim + 2)
+                if self._workspace is None or self._workspace.numel() < need:
+                    self._workspace = torch.empty(need, dtype=torch.float32, device=self.device)
+                part_o = self._workspace
+                part_ml = self._workspace[n * n_heads * n_splits * head_dim:]
+            lib.tis_attention_mfma(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0),
+                                   _ptr(batch.row_seq), _ptr(batch.positions), _ptr(items), n_items, nb, _ptr(out),
+                                   out.stride(0), _ptr(part_o), _ptr(part_ml), n, n_heads, n_kv_heads, head_dim,
+                                   page_size, int(window), float(scale), n_splits, self._stream())
+            return out
         self.attn_generic.tis_attention_generic(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
             _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, head_dim, page_size, int(window),

@@ -44,6 +44,8 @@ class GqaAttention:
         self.w_qkv = to_compute(ops, torch.cat((tensors.of(spec, "q"), tensors.of(spec, "kv")), dim=1).t())
         self.w_o = to_compute(ops, tensors.of(spec, "o").t())
         self.q_width = self.n_heads * self.head_dim
+        if hasattr(ops, "register_attention"):
+            ops.register_attention(self.n_heads, self.n_kv_heads, self.head_dim)
 
     def forward(self, x, ctx, residual=None):
         ops, b = self.ops, ctx.batch

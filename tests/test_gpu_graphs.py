@@ -1,0 +1,66 @@
+"""Captured decode steps against the same steps run kernel by kernel, replay after replay."""
+import pytest
+import torch
+
+import helpers as H
+from tiny_inference_server_amd.engine import Engine
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name", ["C", "D", "A"])
+def test_graph_replays_match_eager_steps(name):
+    """Several requests decode together; each replay is checked against an engine without graphs and against the
+    plain implementation, with eager prompt work and synchronisations between the replays."""
+    folder = H.model_folder(name, "bfloat16")
+    vocab = H.TINY[name]["cfg"].vocab_size
+    reqs = {f"r{i}": H.random_ids(vocab, n, 40 + i) for i, n in enumerate([60, 47, 75])}
+    prompt = 20
+    engines = {flag: Engine(folder, dtype="bfloat16", page_size=H.TINY[name]["page_size"], max_tokens=512,
+                            max_requests=8, use_graphs=flag) for flag in (True, False)}
+    got = {True: {}, False: {}}
+    for flag, eng in engines.items():
+        for rid, ids in reqs.items():
+            eng.step([(rid, ids[:prompt], [])])
+        for p in range(prompt, 47):
+            live = [rid for rid, ids in reqs.items() if p < len(ids)]
+            out = eng.step([(rid, [reqs[rid][p]], [0]) for rid in live])
+            lg = out.logits.float().cpu().clone()
+            for k, rid in enumerate(live):
+                got[flag][(rid, p)] = lg[k]
+            if p % 5 == 0:
+                # eager work of another shape between replays: a new request's prompt, then its end
+                eng.step([("extra", reqs["r0"][:9], [8])])
+                eng.close("extra")
+                torch.cuda.synchronize()
+    assert engines[True].graph_replays >= 20 and engines[False].graph_replays == 0
+    tol = 2e-2 * max(1.0, max(H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values()))
+    H.compare_with_plain(folder, reqs, got[True], {}, tol, 0)
+    H.compare_with_plain(folder, reqs, got[False], {}, tol, 0)
+    # two bfloat16 runs that are each within tol of the plain result are within 2 tol of each other; the graph
+    # cuts the keys into other splits than the eager step, so they are not bit-equal
+    for key in got[False]:
+        assert (got[True][key] - got[False][key]).abs().max().item() <= 2 * tol, key
+
+
+def test_graph_survives_changing_batches():
+    """Requests join and leave: graphs of several shapes are captured and reused; results stay right."""
+    name = "D"
+    folder = H.model_folder(name, "bfloat16")
+    vocab = H.TINY[name]["cfg"].vocab_size
+    reqs = {f"q{i}": H.random_ids(vocab, n, 60 + i) for i, n in enumerate([50, 30, 44, 38])}
+    eng = Engine(folder, dtype="bfloat16", page_size=16, max_tokens=512, max_requests=8)
+    main = {}
+    for rid, ids in reqs.items():
+        eng.step([(rid, ids[:10], [])])
+    fed = {rid: 10 for rid in reqs}
+    while any(fed[r] < len(reqs[r]) for r in reqs):
+        live = [r for r in reqs if fed[r] < len(reqs[r])]
+        out = eng.step([(r, [reqs[r][fed[r]]], [0]) for r in live])
+        lg = out.logits.float().cpu().clone()
+        for k, r in enumerate(live):
+            main[(r, fed[r])] = lg[k]
+            fed[r] += 1
+    assert len(eng._graphs) >= 3 and eng.graph_replays >= 30
+    H.compare_with_plain(folder, reqs, main, {}, 2e-2 * max(1.0, max(
+        H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values())), 0)

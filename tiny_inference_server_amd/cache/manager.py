@@ -64,10 +64,11 @@ class PagePool:
     def check(self) -> None:
         """Every page is either free once or held, never both, never lost."""
         free = list(self._free)
-        if len(set(free)) != len(free):
+        free_set = set(free)
+        if len(free_set) != len(free):
             raise CacheError("a page is on the free list twice")
         for p in range(self.n_pages):
-            if self._held[p] == (p in set(free)):
+            if self._held[p] == (p in free_set):
                 raise CacheError(f"page {p} is {'both held and free' if self._held[p] else 'neither held nor free'}")
 
 

@@ -80,21 +80,51 @@ class _Packer:
         self.total += (a.size + 3) // 4 * 4          # keep every array 16-byte aligned
         return len(self.offsets) - 1
 
-    def upload(self, device) -> List[torch.Tensor]:
-        host = torch.zeros(max(self.total, 4), dtype=torch.int32, pin_memory=(torch.device(device).type == "cuda"))
+    def layout(self):
+        """What must be equal for two packings to share one device buffer."""
+        return tuple(self.offsets)
+
+    def fill(self, host: torch.Tensor) -> None:
         flat = host.numpy()
         for a, (off, _) in zip(self.parts, self.offsets):
             flat[off:off + a.size] = a
-        dev = host.to(device, non_blocking=True)
+
+    def upload(self, device, host: Optional[torch.Tensor] = None, dev: Optional[torch.Tensor] = None):
+        """Copy everything to the device in one transfer; `host` (pinned) and `dev` may be buffers to reuse."""
+        if host is None:
+            host = torch.zeros(max(self.total, 4), dtype=torch.int32,
+                               pin_memory=(torch.device(device).type == "cuda"))
+        self.fill(host)
+        if dev is None:
+            dev = host.to(device, non_blocking=True)
+        else:
+            dev.copy_(host, non_blocking=True)
         out = []
         for a, (off, shape) in zip(self.parts, self.offsets):
             out.append(dev[off:off + a.size].view(shape))
         return out
 
 
+class StepPlan:
+    """A step's arrays on the host, before they are copied to the device."""
+
+    def __init__(self, entries, packer, bt_ids, slots_id, plans):
+        self.entries, self.packer, self.bt_ids, self.slots_id, self.plans = entries, packer, bt_ids, slots_id, plans
+
+    def layout(self):
+        return (self.packer.layout(), tuple(pl["n_rows"] for pl in self.plans),
+                tuple(tuple(sorted((k, v[1:]) for k, v in pl["extra"].items())) for pl in self.plans))
+
+
 def build_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: Sequence[bool], cache, device,
                      max_context: int, plan_rows=None) -> StepBatch:
     """Row arrays for every stage of one step. `cache` is the CacheManager that already covers the new positions."""
+    return materialize(plan_step_batch(entries, lags, has_source, cache, max_context, plan_rows), device)
+
+
+def plan_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: Sequence[bool], cache,
+                    max_context: int, plan_rows=None, table_width: Optional[int] = None) -> StepPlan:
+    """The host half: every array of the step, packed. `table_width` pads the block tables to a fixed width."""
     n_seqs = len(entries)
     pk = _Packer()
     page_size = cache.page_size
@@ -103,6 +133,10 @@ def build_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: 
     bt_ids = {}
     for gname, g in cache.groups.items():
         width = max(1, max(len(g.tables[e.slot]) for e in entries))
+        if table_width is not None:
+            if width > table_width:
+                raise ValueError(f"block tables of {width} pages do not fit the fixed width {table_width}")
+            width = table_width
         tab = np.zeros((n_seqs, width), dtype=np.int32)
         for k, e in enumerate(entries):
             t = g.tables[e.slot]
@@ -170,7 +204,15 @@ def build_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: 
             max_rows=max([n for _, _, n in seq_rows] or [0])))
         prev_rows = seq_rows
 
-    dev = pk.upload(device)
+    return StepPlan(list(entries), pk, bt_ids, slots_id, plans)
+
+
+def materialize(plan: StepPlan, device, host: Optional[torch.Tensor] = None,
+                dev_buffer: Optional[torch.Tensor] = None) -> StepBatch:
+    """The device half: one copy, then views of the device buffer for every array."""
+    entries, pk, bt_ids, slots_id, plans = plan.entries, plan.packer, plan.bt_ids, plan.slots_id, plan.plans
+    n_seqs = len(entries)
+    dev = pk.upload(device, host, dev_buffer)
     tables = {g: dev[i] for g, i in bt_ids.items()}
     stages = []
     for pl in plans:

@@ -15,7 +15,7 @@ from .. import architectures  # noqa: F401  (registers the built-in architecture
 from ..cache.manager import CacheManager, OutOfPages
 from ..config.model_config import ARCHITECTURES, load_config
 from ..weights.loader import load_tensors
-from .batch import Entry, build_step_batch
+from .batch import Entry, build_step_batch, materialize, plan_step_batch
 from .model import Model
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
@@ -39,7 +39,7 @@ class StepOutput:
 class Engine:
     def __init__(self, model_dir: Optional[str] = None, *, config=None, tensors=None, dtype="bfloat16",
                  page_size: int = 16, max_tokens: Optional[int] = None, n_pages: Optional[int] = None,
-                 max_requests: int = 64, device="cuda:0", ops=None):
+                 max_requests: int = 64, device="cuda:0", ops=None, use_graphs: bool = True):
         self.dtype = resolve_dtype(dtype)
         if model_dir is not None:
             config = load_config(model_dir)
@@ -65,6 +65,12 @@ class Engine:
         self.page_size = page_size
         self.cache = CacheManager(self.model.cache_needs(), page_size, n_pages, max_requests, self.dtype, self.device)
         self.requests: Dict[Hashable, Tuple[int, int]] = {}      # id -> (slot, positions fed)
+        # decode steps are replayed from captured graphs where the kernels allow it
+        self.use_graphs = bool(use_graphs) and bool(getattr(ops, "supports_graphs", False))
+        self.graph_table_pages = 64          # block-table widths are rounded up to this many pages
+        self._graphs: Dict[Tuple[int, int], object] = {}
+        self._graph_seen: Dict[Tuple[int, int], int] = {}
+        self.graph_replays = 0
 
     # ---- requests ------------------------------------------------------------------------------------
     def open(self, rid: Hashable) -> None:
@@ -130,12 +136,20 @@ class Engine:
             slot, fed = self.requests[rid]
             self.cache.grow(slot, fed + len(toks))
             batch_entries.append(Entry(slot, fed, list(toks), list(want)))
-        step = build_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache, self.device,
-                                self.spec.max_context, getattr(self.ops, "plan_rows", None))
-        outs = self.model.forward(step, self.cache)
-        n = step.n_wanted
+        logits = None
+        if (self.use_graphs and not heads and
+                all(len(e.tokens) == 1 and e.start >= self.model.max_lag and list(e.want) == [0]
+                    for e in batch_entries)):
+            logits = self._decode_step(batch_entries)
+        if logits is None:
+            step = build_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
+                                    self.device, self.spec.max_context, getattr(self.ops, "plan_rows", None))
+            outs = self.model.forward(step, self.cache)
+        n = sum(len(e.want) for e in batch_entries)
         vocab = self.spec.vocab_size
-        if n:
+        if logits is not None:
+            pass
+        elif n:
             logits = self.model.logits(outs[0].hidden, step.stages[0].want_index, n)
         else:
             logits = torch.empty(0, vocab, dtype=torch.float32, device=self.device)
@@ -157,3 +171,27 @@ class Engine:
             self.requests[rid] = (slot, fed + len(toks))
             self.cache.release_behind(slot, fed + len(toks), self.model.max_lag)
         return StepOutput(logits, head_logits, head_valid)
+
+    def _decode_step(self, batch_entries):
+        """A step of single tokens through a captured graph: logits [requests, vocab], valid until the next step."""
+        from .graph import DecodeGraph
+        pages = max(max(len(g.tables[e.slot]) for e in batch_entries) for g in self.cache.groups.values())
+        width = -(-pages // self.graph_table_pages) * self.graph_table_pages
+        key = (len(batch_entries), width)
+        plan = plan_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
+                               self.spec.max_context, getattr(self.ops, "plan_rows", None), table_width=width)
+        graph = self._graphs.get(key)
+        if graph is None:
+            seen = self._graph_seen.get(key, 0)
+            self._graph_seen[key] = seen + 1
+            if seen == 0:
+                # the first step of a shape runs as it is: it warms the library's choices for these shapes and
+                # sizes the kernels' workspace, so the capture that follows records kernel launches only
+                step = materialize(plan, self.device)
+                for st in step.stages:
+                    st.max_kv_len = width * self.page_size
+                outs = self.model.forward(step, self.cache)
+                return self.model.logits(outs[0].hidden, step.stages[0].want_index, len(batch_entries))
+            graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size)
+        self.graph_replays += 1
+        return graph.run(plan)

@@ -106,7 +106,7 @@ class Scheduler:
         total = self.engine.total_pages()
         # pages are only taken when a request runs, so the free count does not move while admitting: keep a
         # budget instead (the reference's fix, server.py:143-147)
-        budget = self.engine.free_pages() - sum(self._grow_pages(r, 1) for r in self.active)
+        budget = self.engine.free_pages() - sum(self._grow_pages(r, len(r.ids) - r.fed) for r in self.active)
         while self.queue and len(self.active) < self.max_batch:
             q = self.queue[0]
             need_now = pages_for(len(q.ids), self.page_size)

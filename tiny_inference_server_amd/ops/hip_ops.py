@@ -92,6 +92,7 @@ def library(name: str) -> _Lib:
 
 # wavefronts the attention launch aims for, so that short batches still spread over the chip
 _ATTN_TARGET_WAVES = 1024
+_ATTN_WORKSPACE_FLOATS = 16 << 20
 
 
 def attention_items(seq_rows, group_size: int):
@@ -121,6 +122,7 @@ def _rows_view(t: torch.Tensor, what: str):
 
 class HipOps:
     """The operations of one engine instance: a device, a compute dtype, and the kernels for them."""
+    supports_graphs = True      # every launch goes to torch's current stream, so a stream capture records it
 
     def __init__(self, device="cuda:0", dtype=torch.bfloat16):
         if dtype not in _DT:
@@ -367,11 +369,15 @@ class HipOps:
             if lib is None:
                 lib = self._attn_mfma[head_dim] = library(f"attention_mfma@{head_dim}")
             n_splits = max(1, min(-(-_ATTN_TARGET_WAVES // (n_items * n_kv_heads)), -(-batch.max_kv_len // 64)))
+            # partial results of split key ranges live in one workspace of fixed size, allocated once and never
+            # moved (captured graphs hold its address); fewer splits where it would not suffice
+            n_splits = max(1, min(n_splits, _ATTN_WORKSPACE_FLOATS // (n * n_heads * (head_dim + 2))))
             part_o = part_ml = None
             if n_splits > 1:
-                need = n * n_heads * n_splits * (head_dim + 2)
-                if self._workspace is None or self._workspace.numel() < need:
-                    self._workspace = torch.empty(need, dtype=torch.float32, device=self.device)
+                if self._workspace is None:
+                    if torch.cuda.is_current_stream_capturing():
+                        raise KernelError("the attention workspace must exist before a graph is captured")
+                    self._workspace = torch.empty(_ATTN_WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
                 part_o = self._workspace
                 part_ml = self._workspace[n * n_heads * n_splits * head_dim:]
             lib.tis_attention_mfma(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0),

@@ -1,0 +1,118 @@
+"""Generation through the entry points on the GPU, and the replay program as a user runs it."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import plain_model as pm
+from tiny_inference_server_amd.engine.generate import generate
+from tiny_inference_server_amd.sampling import SamplingParams, uniform_for
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_equals_plain(name):
+    """BASELINE's tiny workloads: 3 prompts of 5/17/33 tokens, 16 greedy tokens each (A); 1/9/24/40 (B)."""
+    folder = H.model_folder(name, "float32")
+    cfg, w = pm.read_model_folder(folder)
+    lens = [5, 17, 33] if name == "A" else [1, 9, 24, 40]
+    prompts = [H.random_ids(cfg["vocab"], n, 90 + i) for i, n in enumerate(lens)]
+    want = [pm.greedy_generate(p, 16, w, cfg) for p in prompts]
+    ps = H.TINY[name]["page_size"]
+    assert generate(folder, prompts, max_new_tokens=16, temperature=0.0, dtype="float32", tokens_per_block=ps) == want
+    # portions under a small token budget, few pages, preemption allowed: the same tokens
+    got, s = generate(folder, prompts, max_new_tokens=16, temperature=0.0, dtype="float32", tokens_per_block=ps,
+                      max_batch=2, token_budget=9, plan="cur", pool_tokens=5 * 16, return_scheduler=True)
+    assert got == want and s.engine.free_pages() == s.engine.total_pages()
+
+
+def test_bfloat16_generation_follows_the_plain_choice_where_it_is_clear():
+    """In bfloat16 an arg-max may flip where two logits are close; where the plain model's margin is wide it must not."""
+    folder = H.model_folder("D", "bfloat16")
+    cfg, w = pm.read_model_folder(folder)
+    prompts = [H.random_ids(cfg["vocab"], n, 95 + i) for i, n in enumerate([12, 30])]
+    got = generate(folder, prompts, max_new_tokens=12, temperature=0.0, dtype="bfloat16")
+    for p, g in zip(prompts, got):
+        ids = list(p)
+        for t in g:
+            lg = pm.logits_of(pm.trunk_hidden(ids, w, cfg)[-1:], w, cfg)[0]
+            top2 = torch.topk(lg, 2).values
+            if (top2[0] - top2[1]).item() > 0.1:
+                assert t == int(lg.argmax())
+            ids.append(t)
+
+
+def test_temperature_sampling_with_seeded_streams():
+    """Tiny B's workload: temperature 0.8, seed 0, mixed chunked prefill and decode; token by token the draw is the
+    plain rule's (server.py:22-50) on the plain logits with the request's own uniform number."""
+    folder = H.model_folder("B", "float32")
+    cfg, w = pm.read_model_folder(folder)
+    prompts = [H.random_ids(cfg["vocab"], n, 97 + i) for i, n in enumerate([1, 9, 24, 40])]
+    params = [SamplingParams(max_new_tokens=8, temperature=0.8, seed=i) for i in range(4)]
+    got = generate(folder, prompts, params=params, dtype="float32", tokens_per_block=8, token_budget=16, max_batch=4)
+    for p, sp, g in zip(prompts, params, got):
+        ids = list(p)
+        for i in range(8):
+            lg = pm.logits_of(pm.trunk_hidden(ids, w, cfg)[-1:], w, cfg)[0]
+            probs = pm.sampling_probs(lg, sp.temperature)
+            u = uniform_for(sp.seed, i)
+            c = torch.cumsum(probs, 0)
+            want = pm.pick_by_uniform(probs, u)
+            # a draw that lands within rounding of a boundary of the cumulative distribution may go either way
+            near = (c - u).abs().min().item() < 1e-5
+            assert g[i] == want or near, (i, g[i], want)
+            ids.append(g[i])
+
+
+def test_command_line_runs(tmp_path):
+    folder = H.model_folder("A", "bfloat16")
+    out = subprocess.run([sys.executable, "-m", "tiny_inference_server_amd", "--model", folder, "--prompt-ids", "5,17,3",
+                          "--prompt-ids", "9", "--max-new-tokens", "5", "--greedy", "--pool-bytes", "1MiB"],
+                         cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [l for l in out.stdout.splitlines() if l.startswith("OUTPUT:")]
+    assert len(lines) == 2 and all(len(l.split()) == 6 for l in lines)
+    assert "tok/s" in out.stdout
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 2e-2)])
+def test_replay_program(tmp_path, dtype, tol):
+    """bin/trace_run as a subprocess: mixed steps with so few pages that they are used again."""
+    name = "C"
+    folder = H.model_folder(name, "float32" if dtype == "float32" else "bfloat16")
+    vocab = H.TINY[name]["cfg"].vocab_size
+    reqs = {f"r{i}": H.random_ids(vocab, n, 70 + i) for i, n in enumerate([40, 64, 30, 70, 12, 50])}
+    steps, peak = H.mixed_trace(reqs, max_live=4, seed=8)
+    out_dir = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out_dir), "--max-tokens", str(peak), "--heads"],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert proc.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+    fed = {r: 0 for r in reqs}
+    worst = 0.0
+    scale = max(1.0, max(H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values()))
+    for s in steps:
+        wanted = sum(len(e["want"]) for e in s["entries"])
+        arr = np.fromfile(out_dir / f"{s['step']}.f32", dtype="<f4").reshape(wanted, vocab)
+        h0 = np.fromfile(out_dir / f"{s['step']}.head0.f32", dtype="<f4").reshape(wanted, vocab)
+        row = 0
+        for e in s["entries"]:
+            main, heads = H.plain_logits(folder, reqs[e["id"]])
+            for i in e["want"]:
+                p = fed[e["id"]] + i
+                worst = max(worst, np.abs(arr[row] - main[p].numpy()).max())
+                if p - 1 >= 0:
+                    worst = max(worst, np.abs(h0[row] - heads[0][p - 1].numpy()).max())
+                else:
+                    assert np.isnan(h0[row]).all()
+                row += 1
+            fed[e["id"]] += len(e["tokens"])
+    assert worst <= tol * scale

@@ -1,0 +1,206 @@
+"""Each part alone on the GPU against the plain implementation's function for it, and a toy mixer with state of
+its own that is registered, built and stepped from here without touching the framework's files."""
+import math
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+import helpers as H
+import plain_model as pm
+from tiny_inference_server_amd.cache import CacheManager
+from tiny_inference_server_amd.config import ARCHITECTURES, Architecture
+from tiny_inference_server_amd.engine import Engine
+from tiny_inference_server_amd.engine.batch import Entry, build_step_batch
+from tiny_inference_server_amd.parts import (ARRANGEMENTS, MIXERS, CallContext, LayerCall, LayerSpec, ModelSpec, PartSpec,
+                                             StageSpec, StateNeed, Tensors, build_part, to_compute)
+from tiny_inference_server_amd.weights import random_tensors
+
+pytestmark = pytest.mark.gpu
+
+DT = [("float32", torch.float32, 2e-5), ("bfloat16", torch.bfloat16, 3e-2)]
+
+
+def ops_of(dtype):
+    from tiny_inference_server_amd.ops.hip_ops import HipOps
+    return HipOps("cuda:0", dtype)
+
+
+def rnd(shape, seed, scale=1.0):
+    return scale * torch.randn(shape, generator=torch.Generator().manual_seed(seed))
+
+
+@pytest.mark.parametrize("name,dtype,tol", DT)
+def test_norm_part(name, dtype, tol):
+    ops = ops_of(dtype)
+    gain = (1 + 0.1 * rnd((200,), 1)).to(dtype)
+    part = build_part(PartSpec("norm", "rmsnorm_l2", {"width": 200, "eps": 1e-5}, {"gain": "g"}), Tensors({"g": gain}), ops)
+    x = rnd((7, 200), 2, 3.0).to(dtype)
+    want = pm.rms_norm(x.double(), gain.double(), 1e-5)
+    assert (part(x.cuda()).cpu().double() - want).abs().max() <= tol * want.abs().max()
+
+
+def test_rotary_part_table():
+    ops = ops_of(torch.float32)
+    part = build_part(PartSpec("position", "rotary", {"head_dim": 48, "base": 5e5, "max_context": 300, "pairing": "half"}),
+                      Tensors({}), ops)
+    table, interleaved = part.rotary()
+    cos, sin = pm.rope_tables(300, 48, 5e5)
+    assert not interleaved and table.shape == (300, 24, 2)
+    torch.testing.assert_close(table[..., 0].cpu().double(), cos[:, :24], atol=2e-5, rtol=0)      # angles up to 300 in 32-bit
+    torch.testing.assert_close(table[..., 1].cpu().double(), sin[:, :24], atol=2e-5, rtol=0)
+    with pytest.raises(ValueError, match="pairing"):
+        build_part(PartSpec("position", "rotary", {"head_dim": 8, "base": 1e4, "max_context": 8, "pairing": "odd"}), Tensors({}), ops)
+
+
+@pytest.mark.parametrize("name,dtype,tol", DT)
+def test_feed_forward_part(name, dtype, tol):
+    ops = ops_of(dtype)
+    D, Fh = 96, 200
+    t = {"g": rnd((D, Fh), 3, D ** -0.5).to(dtype), "u": rnd((D, Fh), 4, D ** -0.5).to(dtype), "d": rnd((Fh, D), 5, Fh ** -0.5).to(dtype)}
+    part = build_part(PartSpec("feed_forward", "swiglu", {"d_model": D, "hidden": Fh}, {"gate": "g", "up": "u", "down": "d"}),
+                      Tensors(t), ops)
+    x, res = rnd((9, D), 6).to(dtype), rnd((9, D), 7).to(dtype)
+    want = res.double() + pm.swiglu_ffn(x.double(), t["g"].double(), t["u"].double(), t["d"].double())
+    got = part.forward(x.cuda(), residual=res.cuda()).cpu().double()
+    assert (got - want).abs().max() <= tol * want.abs().max()
+
+
+def one_sequence_batch(needs, n_rows, page_size, dtype, start=0):
+    cache = CacheManager(needs, page_size, 16, 2, dtype, torch.device("cuda:0"))
+    slot = cache.open_request()
+    cache.grow(slot, start + n_rows)
+    step = build_step_batch([Entry(slot, start, list(range(n_rows)), [])], [0], [False], cache, torch.device("cuda:0"), 4096)
+    return cache, step.stages[0]
+
+
+@pytest.mark.parametrize("name,dtype,tol", DT)
+@pytest.mark.parametrize("n_heads,n_kv,hd", [(4, 2, 16), (3, 1, 32), (6, 2, 8)])
+def test_attention_mixer_and_block(name, dtype, tol, n_heads, n_kv, hd):
+    ops = ops_of(dtype)
+    D, Fh, T, eps, base = n_heads * hd, 72, 21, 1e-6, 1000.0
+    pos = PartSpec("position", "rotary", {"head_dim": hd, "base": base, "max_context": 64, "pairing": "half"})
+    mixer = PartSpec("mixer", "gqa_attention", {"d_model": D, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd,
+                                                "window": 0, "position": pos},
+                     {"q": "b.att.q_proj.weight", "kv": "b.att.kv_proj.weight", "o": "b.att.linear_proj.weight"})
+    norm = lambda n: PartSpec("norm", "rmsnorm_l2", {"width": D, "eps": eps}, {"gain": n})
+    ffn = PartSpec("feed_forward", "swiglu", {"d_model": D, "hidden": Fh},
+                   {"gate": "b.ffn.swig.linear1.weight", "up": "b.ffn.swig.linear2.weight", "down": "b.ffn.fc.weight"})
+    layer = LayerSpec("prenorm_residual", mixer, norm("b.att.rms_norm_att.scale"), ffn, norm("b.rms_norm_ffn.scale"))
+    t = {"b.att.q_proj.weight": rnd((D, D), 10, D ** -0.5), "b.att.kv_proj.weight": rnd((D, 2 * n_kv * hd), 11, D ** -0.5),
+         "b.att.linear_proj.weight": rnd((D, D), 12, D ** -0.5), "b.ffn.swig.linear1.weight": rnd((D, Fh), 13, D ** -0.5),
+         "b.ffn.swig.linear2.weight": rnd((D, Fh), 14, D ** -0.5), "b.ffn.fc.weight": rnd((Fh, D), 15, Fh ** -0.5),
+         "b.att.rms_norm_att.scale": 1 + 0.1 * rnd((D,), 16), "b.rms_norm_ffn.scale": 1 + 0.1 * rnd((D,), 17)}
+    t = {k: v.to(dtype) for k, v in t.items()}
+    block = ARRANGEMENTS.get("prenorm_residual")(layer, Tensors(t), ops)
+    need = block.mixer.cache_need(mixer.params)
+    cache, b = one_sequence_batch({"k": need}, T, 16, dtype)
+    group = cache.group_of["k"]
+    ctx = CallContext(batch=b, group=group, plane=cache.groups[group].plane("k"))
+    x = rnd((T, D), 18).to(dtype)
+    cfg = {"n_heads": n_heads, "group": n_heads // n_kv, "eps": eps, "base": base}
+    w64 = {k: v.double() for k, v in t.items()}
+    want = pm.block(x.double(), w64, "b.", cfg, torch.arange(T))
+    got = block.forward(x.cuda(), ctx).cpu().double()
+    assert (got - want).abs().max() <= tol * want.abs().max()
+    # the mixer alone: out = attention(norm'd input) . Wo + residual
+    a = pm.rms_norm(x.double(), w64["b.att.rms_norm_att.scale"], eps)
+    q = pm.apply_rope((a @ w64["b.att.q_proj.weight"]).view(T, n_heads, hd), torch.arange(T), base)
+    kv = (a @ w64["b.att.kv_proj.weight"]).view(T, 2, n_kv, hd)
+    k = pm.apply_rope(kv[:, 0], torch.arange(T), base)
+    o = pm.causal_gqa_attention(q, k, kv[:, 1], n_heads // n_kv).reshape(T, D) @ w64["b.att.linear_proj.weight"]
+    got = block.mixer.forward(a.to(dtype).cuda(), ctx).cpu().double()
+    assert (got - o).abs().max() <= tol * max(1.0, o.abs().max())
+
+
+# ---- a toy mixer with state of its own, and a toy architecture around it, all defined here -------------------------
+
+@MIXERS.register("toy_decay", replace=True)
+class ToyDecayMixer:
+    """s <- decay * s + x for every row in order; y = s . W (+ residual). Its state is one vector per request."""
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        return {"w": (params["d_model"], params["d_model"])}
+
+    @classmethod
+    def cache_need(cls, params):
+        return StateNeed((params["d_model"],), "float32")
+
+    def __init__(self, spec, tensors, ops):
+        self.ops, self.decay = ops, float(spec.params["decay"])
+        self.w = to_compute(ops, tensors.of(spec, "w").t())
+
+    def forward(self, x, ctx, residual=None):
+        s_all = torch.empty(x.shape[0], x.shape[1], dtype=torch.float32, device=x.device)
+        for (first, p0, n), slot in zip(ctx.batch.seq_rows, ctx.batch.host_slots):
+            s = ctx.state[slot]
+            for r in range(first, first + n):
+                s = self.decay * s + x[r].float()
+                s_all[r] = s
+            if n:
+                ctx.state[slot] = s
+        return self.ops.linear(s_all.to(x.dtype), self.w, residual=residual)
+
+
+@dataclass(frozen=True)
+class ToyConfig:
+    d_model: int
+    vocab_size: int
+    hidden: int
+    decay: float
+    max_context: int = 128
+    architecture: str = "ToyStateModel"
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw["d_model"], raw["vocab_size"], raw["hidden"], raw["decay"], raw.get("max_context", 128))
+
+    def to_dict(self):
+        return dict(self.__dict__)
+
+
+def toy_spec(cfg):
+    norm = lambda n: PartSpec("norm", "rmsnorm_l2", {"width": cfg.d_model, "eps": 1e-6}, {"gain": n})
+    layers = []
+    for l in range(2):
+        mixer = PartSpec("mixer", "toy_decay", {"d_model": cfg.d_model, "decay": cfg.decay}, {"w": f"l{l}.mix.w"})
+        ffn = PartSpec("feed_forward", "swiglu", {"d_model": cfg.d_model, "hidden": cfg.hidden},
+                       {"gate": f"l{l}.g", "up": f"l{l}.u", "down": f"l{l}.d"})
+        layers.append(LayerSpec("prenorm_residual", mixer, norm(f"l{l}.n1"), ffn, norm(f"l{l}.n2")))
+    # the run order is data: layer 0, layer 1, then layer 0 again with a state of its own
+    stage = StageSpec("trunk", 0, PartSpec("stage_input", "token_embedding"),
+                      (LayerCall(0), LayerCall(1), LayerCall(0)), norm("out"))
+    return ModelSpec(cfg.d_model, cfg.vocab_size, cfg.max_context, tuple(layers), (stage,), "emb", "emb")
+
+
+def toy_plain(ids, w, cfg):
+    x = w["emb"][torch.tensor(ids)].double()
+    for l in (0, 1, 0):
+        a = pm.rms_norm(x, w[f"l{l}.n1"].double(), 1e-6)
+        s, rows = torch.zeros(cfg.d_model, dtype=torch.float64), []
+        for r in range(len(ids)):
+            s = cfg.decay * s + a[r]
+            rows.append(s)
+        x = x + torch.stack(rows) @ w[f"l{l}.mix.w"].double()
+        x = x + pm.swiglu_ffn(pm.rms_norm(x, w[f"l{l}.n2"].double(), 1e-6), w[f"l{l}.g"].double(), w[f"l{l}.u"].double(),
+                              w[f"l{l}.d"].double())
+    return pm.rms_norm(x, w["out"].double(), 1e-6) @ w["emb"].double().T
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped():
+    ARCHITECTURES.register("ToyStateModel", Architecture("ToyStateModel", ToyConfig, toy_spec), replace=True)
+    cfg = ToyConfig(d_model=48, vocab_size=101, hidden=80, decay=0.7)
+    w = random_tensors(cfg, 9, std=0.1, gain_jitter=0.1, dtype="float32")
+    eng = Engine(config=cfg, tensors=w, dtype="float32", page_size=16, max_tokens=64, max_requests=3)
+    assert sorted(eng.model.cache_needs()) == ["trunk.0", "trunk.1", "trunk.2"] and not eng.cache.groups
+    reqs = {"a": H.random_ids(101, 23, 1), "b": H.random_ids(101, 9, 2)}
+    main = {}
+    # whole, then in portions beside each other, then a slot used again by a new request
+    for trace in (H.whole_trace(reqs), H.mixed_trace(reqs, 2, 3)[0], H.portions_trace({"b": reqs["b"]}, 1)):
+        got, _ = H.run_trace(eng, trace, heads=False)
+        for (rid, p), lg in got.items():
+            want = toy_plain(reqs[rid], w, cfg)[p]
+            assert (lg.double() - want).abs().max() <= 2e-5 * max(1.0, want.abs().max()), (rid, p)
+    ARCHITECTURES.unregister("ToyStateModel")
+    MIXERS.unregister("toy_decay")

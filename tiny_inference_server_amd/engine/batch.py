@@ -54,6 +54,7 @@ class StageBatch:
     max_kv_len: int
     max_seq_rows: int
     seq_rows: List[Tuple[int, int, int]]      # host copy: (first row, first position, rows) per entry
+    host_slots: List[int] = field(default_factory=list)       # host copy: state slot per entry
     extras: Dict[str, object] = field(default_factory=dict)   # what faster kernels plan on the host
 
 
@@ -225,5 +226,6 @@ def materialize(plan: StepPlan, device, host: Optional[torch.Tensor] = None,
             keep_slot=dev[pl["keep_slot"]] if pl["keep_slot"] is not None else None,
             keep_count=pl["keep_count"], want_index=dev[pl["want"]], want_valid=pl["valid"],
             max_kv_len=pl["max_kv"], max_seq_rows=pl["max_rows"], seq_rows=pl["seq_rows"],
+            host_slots=[e.slot for e in entries],
             extras={k: (dev[v[0]],) + tuple(v[1:]) for k, v in pl["extra"].items()}))
     return StepBatch(list(entries), stages, sum(len(e.want) for e in entries))

@@ -66,7 +66,7 @@ class Engine:
         self.cache = CacheManager(self.model.cache_needs(), page_size, n_pages, max_requests, self.dtype, self.device)
         self.requests: Dict[Hashable, Tuple[int, int]] = {}      # id -> (slot, positions fed)
         # decode steps are replayed from captured graphs where the kernels allow it
-        self.use_graphs = bool(use_graphs) and bool(getattr(ops, "supports_graphs", False))
+        self.use_graphs = bool(use_graphs) and bool(getattr(ops, "supports_graphs", False)) and self.model.graph_safe
         self.graph_table_pages = 64          # block-table widths are rounded up to this many pages
         self._graphs: Dict[Tuple[int, int], object] = {}
         self._graph_seen: Dict[Tuple[int, int], int] = {}
@@ -175,7 +175,7 @@ class Engine:
     def _decode_step(self, batch_entries):
         """A step of single tokens through a captured graph: logits [requests, vocab], valid until the next step."""
         from .graph import DecodeGraph
-        pages = max(max(len(g.tables[e.slot]) for e in batch_entries) for g in self.cache.groups.values())
+        pages = max((max(len(g.tables[e.slot]) for e in batch_entries) for g in self.cache.groups.values()), default=1)
         width = -(-pages // self.graph_table_pages) * self.graph_table_pages
         key = (len(batch_entries), width)
         plan = plan_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,

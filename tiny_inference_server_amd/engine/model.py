@@ -29,6 +29,12 @@ class Model:
         emb = to_compute(ops, tensors[spec.embedding])
         self.shared = {"embedding": emb,
                        "lm_head": emb if spec.lm_head == spec.embedding else to_compute(ops, tensors[spec.lm_head])}
+        # a step may be captured as a graph only if every part promises that what it launches depends on the
+        # step's device arrays alone, never on host values that change from step to step
+        parts = list(self.inputs) + list(self.out_norms)
+        for blk in self.layers:
+            parts += [getattr(blk, n) for n in ("mixer", "mixer_norm", "ffn", "ffn_norm") if hasattr(blk, n)] or [blk]
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
         self.lags = [st.lag for st in spec.stages]
         self.max_lag = max(self.lags)
         self.reads_previous = [bool(getattr(part_class(st.input), "reads_previous", False)) for st in spec.stages]

@@ -20,6 +20,7 @@ class GqaAttention:
     tensors: q (d_model, n_heads*head_dim), kv (d_model, 2*n_kv_heads*head_dim) with the key columns first,
     o (n_heads*head_dim, d_model); all stored [in, out] as the reference applies them (x @ W).
     """
+    graph_safe = True
 
     @classmethod
     def tensor_shapes(cls, params):

@@ -14,6 +14,9 @@ norm            __call__(x) -> y                       rows in, rows out
 position        rotary() -> (table | None, interleaved)   a table of (cos, sin) per position and pair for
                                                        mixers that rotate queries and keys; and
                 on_embedding(x, batch) -> x            a hook for encodings that act on the embedded rows
+every part      graph_safe = True                      class attribute, only if what the part launches depends on the
+                                                       step's device arrays alone (then decode steps may be captured
+                                                       as graphs); absent or False keeps the model on plain launches
 mixer           cache_need(params) -> PagedKvNeed | StateNeed | None      classmethod
                 forward(x, ctx, residual=None) -> y    x: normed rows; ctx: CallContext; adds `residual` if given
 feed-forward    forward(x, residual=None) -> y

@@ -13,6 +13,7 @@ class SwiGlu:
     params: d_model, hidden. tensors: gate (d_model, hidden), up (d_model, hidden), down (hidden, d_model),
     stored [in, out].
     """
+    graph_safe = True
 
     @classmethod
     def tensor_shapes(cls, params):

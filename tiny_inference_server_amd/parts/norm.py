@@ -11,6 +11,7 @@ class RmsNormL2:
     The reference's norm (main_models_new.py:31-42): the L2 norm of the row with eps added to the norm
     itself, not under the root. params: width, eps. tensors: gain (width,).
     """
+    graph_safe = True
 
     @classmethod
     def tensor_shapes(cls, params):

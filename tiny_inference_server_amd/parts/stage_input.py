@@ -10,6 +10,7 @@ from .spec import StateNeed
 @STAGE_INPUTS.register("token_embedding")
 class TokenEmbedding:
     """x = E[token] (reference main_models_new.py:199)."""
+    graph_safe = True
 
     @classmethod
     def tensor_shapes(cls, params):
@@ -38,6 +39,7 @@ class FusePreviousStage:
 
     params: d_model, embed_norm (a PartSpec). tensors: proj (2*d_model, d_model), stored [in, out].
     """
+    graph_safe = True
     reads_previous = True
 
     @classmethod

@@ -132,6 +132,8 @@ class HipOps:
         self.device = torch.device(device)
         self.dtype = dtype
         self.code = _DT[dtype]
+        # whatever is not built yet is compiled side by side, not one after the other
+        _build.build(["rowwise", "rope_cache", "attention_generic", "gemm_plain", "sampling"])
         self.rowwise = library("rowwise")
         self.rope = library("rope_cache")
         self.attn_generic = library("attention_generic")

@@ -53,19 +53,23 @@ class TorchOps:
         dst[dst_index.long()] = src[src_index.long()]
 
     def swiglu(self, gu, out=None):
-        F = gu.shape[1] // 2
-        g, u = gu[:, :F].float(), gu[:, F:].float()
+        g, u = gu[:, 0::2].float(), gu[:, 1::2].float()      # gate and up columns come interleaved
         y = (g * torch.sigmoid(g) * u).to(gu.dtype)
         if out is not None:
             out.copy_(y)
             return out
         return y
 
-    def linear(self, x, w, residual=None, out_dtype=None):
+    def linear(self, x, w, residual=None, out_dtype=None, rms=None):
+        if rms is not None:
+            x = self.rmsnorm(x, rms[0], rms[1])
         y = x.float() @ w.float().t()
         if residual is not None:
             y = y + residual.float()
         return y.to(out_dtype or self.dtype)
+
+    def linear_swiglu(self, x, w, rms=None):
+        return self.swiglu(self.linear(x, w, rms=rms))
 
     # ---- rotary + cache write ---------------------------------------------------------------------------
     def rope_write_kv(self, qkv, positions, write_slots, table, plane, n_heads, n_kv_heads, head_dim, page_size,

@@ -101,37 +101,58 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     for (int db = 0; db < DB; ++db) o[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int s = s_begin; s < s_end; ++s) {
-    const int kb = k_lo + s * 32;
-    // page and first slot of the two 16-key tiles; a tile past the item's last key is skipped
-    bool tile_ok[2];
-    const bf16* kp[2];
-    const bf16* vp[2];
+  // One step's keys and values in registers. A step's loads are all issued together, one step ahead of the
+  // products that use them, and the page ids two steps ahead, so that a wave always has a step's worth of
+  // requests in flight instead of waiting out a chain of dependent loads per step.
+  struct Tiles {
+    bf16x8 k[2][DC];
+    bf16x8 v[DB];
+    bool ok[2];
+  };
+  auto page_ids = [&](int s, int (&pg)[2]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const int key0 = kb + t * 16;
-      tile_ok[t] = key0 < k_hi;
-      const long page = tile_ok[t] ? bt[key0 / page_size] : 0;
-      const int slot0 = key0 % page_size;
-      kp[t] = plane + page * page_stride + k_head + (long)(slot0 + c16) * HD + g * 8;
-      vp[t] = plane + page * page_stride + v_head + (long)c16 * page_size + slot0 + g * 4;
+      const int key0 = k_lo + s * 32 + t * 16;
+      pg[t] = (s < s_end && key0 < k_hi) ? bt[key0 / page_size] : -1;
     }
+  };
+  auto load_tiles = [&](int s, const int (&pg)[2], Tiles& T) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key0 = k_lo + s * 32 + t * 16;
+      const int slot0 = key0 % page_size;
+      T.ok[t] = pg[t] >= 0;
+      const bf16* base = plane + (long)(T.ok[t] ? pg[t] : 0) * page_stride;
+      const bf16* kp = base + k_head + (long)(slot0 + c16) * HD + g * 8;
+      const bf16* vp = base + v_head + (long)c16 * page_size + slot0 + g * 4;
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) {
+        bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (T.ok[t] && dc * 32 + g * 8 < HD) ka = load8(kp + dc * 32);
+        T.k[t][dc] = ka;
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        bf16x4 h = {0, 0, 0, 0};
+        if (T.ok[t]) h = load4(vp + (long)db * 16 * page_size);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) T.v[db][t * 4 + e] = h[e];
+      }
+    }
+  };
+  auto consume = [&](int s, const Tiles& T) {
+    const int kb = k_lo + s * 32;
     // S^T = K . Q^T
     f32x4 st[2][NB];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) st[t][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-      if (tile_ok[t]) {
 #pragma unroll
-        for (int dc = 0; dc < DC; ++dc) {
-          bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (dc * 32 + g * 8 < HD) ka = load8(kp[t] + dc * 32);
+      for (int dc = 0; dc < DC; ++dc)
 #pragma unroll
-          for (int nb = 0; nb < NB; ++nb)
-            st[t][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[nb][dc], st[t][nb], 0, 0, 0);
-        }
-      }
+        for (int nb = 0; nb < NB; ++nb)
+          st[t][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(T.k[t][dc], qb[nb][dc], st[t][nb], 0, 0, 0);
     }
     // mask, running maximum and sum per column, P in bfloat16 as the B operand of the second product
     bf16x8 pb[NB];
@@ -145,7 +166,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = kb + t * 16 + g * 4 + i;
-          const bool ok = tile_ok[t] && key <= col_pos[nb] && key >= col_lo[nb];
+          const bool ok = T.ok[t] && key <= col_pos[nb] && key >= col_lo[nb];
           const float v = ok ? st[t][nb][i] * scale_log2 : -INFINITY;
           sv[t * 4 + i] = v;
           tmax = fmaxf(tmax, v);
@@ -169,21 +190,32 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     }
     // O^T = O^T * alpha + V^T . P^T
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      bf16x8 va;
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        bf16x4 h = {0, 0, 0, 0};
-        if (tile_ok[t]) h = load4(vp[t] + (long)db * 16 * page_size);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) va[t * 4 + e] = h[e];
-      }
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         f32x4 acc = o[nb][db];
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] *= alpha[nb];
-        o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[nb], acc, 0, 0, 0);
+        o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(T.v[db], pb[nb], acc, 0, 0, 0);
+      }
+  };
+
+  if (s_begin < s_end) {
+    Tiles ta, tb;
+    int pa[2], pn[2];
+    page_ids(s_begin, pa);
+    page_ids(s_begin + 1, pn);
+    load_tiles(s_begin, pa, ta);
+    for (int s = s_begin; s < s_end; s += 2) {
+      // pn holds the page ids of step s+1
+      int pq[2];
+      page_ids(s + 2, pq);
+      if (s + 1 < s_end) load_tiles(s + 1, pn, tb);
+      consume(s, ta);
+      if (s + 1 < s_end) {
+        page_ids(s + 3, pn);
+        if (s + 2 < s_end) load_tiles(s + 2, pq, ta);
+        consume(s + 1, tb);
       }
     }
   }
@@ -216,27 +248,54 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
 }
 
 // out[row, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s      (reference paged_attention_kernels.py:121-204)
-__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ part_o,
-                                                             const float2* __restrict__ part_ml,
-                                                             bf16* __restrict__ out, long out_ld, int n_heads,
-                                                             int n_splits) {
+// Four groups of 64 lanes take the splits in turn, a lane holding up to four outputs; the groups' sums meet in
+// LDS and are added in a fixed order. All loads of a lane are independent, so they overlap.
+static constexpr int MG = 4;             // split groups per workgroup
+static constexpr int MD = (HD + 63) / 64;  // outputs per lane
+
+__global__ __launch_bounds__(MG * 64) void attention_merge_kernel(const float* __restrict__ part_o,
+                                                                  const float2* __restrict__ part_ml,
+                                                                  bf16* __restrict__ out, long out_ld, int n_heads,
+                                                                  int n_splits) {
+  __shared__ float so[MG][MD][64];
+  __shared__ float sl[MG];
   const long row = blockIdx.x;
   const int head = blockIdx.y;
+  const int grp = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long base = (row * n_heads + head) * n_splits;
   float M = -INFINITY;
   for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[base + s].x);
+  float acc[MD];
+#pragma unroll
+  for (int j = 0; j < MD; ++j) acc[j] = 0.f;
   float L = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
+  for (int s = grp; s < n_splits; s += MG) {
     const float2 ml = part_ml[base + s];
-    if (ml.x > -INFINITY) L += exp2f(ml.x - M) * ml.y;
-  }
-  for (int d = threadIdx.x; d < HD; d += 64) {
-    float acc = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float mx = part_ml[base + s].x;
-      if (mx > -INFINITY) acc += exp2f(mx - M) * part_o[(base + s) * HD + d];
+    if (ml.x == -INFINITY) continue;     // a split that held no key of this row
+    const float w = exp2f(ml.x - M);
+    L += w * ml.y;
+#pragma unroll
+    for (int j = 0; j < MD; ++j) {
+      const int d = j * 64 + lane;
+      if (d < HD) acc[j] += w * part_o[(base + s) * HD + d];
     }
-    out[row * out_ld + (long)head * HD + d] = static_cast<__bf16>(acc / L);
+  }
+#pragma unroll
+  for (int j = 0; j < MD; ++j) so[grp][j][lane] = acc[j];
+  if (lane == 0) sl[grp] = L;
+  __syncthreads();
+  if (grp != 0) return;
+  float Lt = sl[0];
+#pragma unroll
+  for (int gq = 1; gq < MG; ++gq) Lt += sl[gq];
+#pragma unroll
+  for (int j = 0; j < MD; ++j) {
+    const int d = j * 64 + lane;
+    if (d >= HD) continue;
+    float t = so[0][j][lane];
+#pragma unroll
+    for (int gq = 1; gq < MG; ++gq) t += so[gq][j][lane];
+    out[row * out_ld + (long)head * HD + d] = static_cast<__bf16>(t / Lt);
   }
 }
 
@@ -277,7 +336,7 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
   if (rc) return rc;
   if (n_splits > 1) {
     dim3 mgrid(rows, n_heads);
-    attention_merge_kernel<<<mgrid, 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld, n_heads,
+    attention_merge_kernel<<<mgrid, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld, n_heads,
                                                      n_splits);
     rc = tis_launch_status("attention_merge");
   }

@@ -1,0 +1,202 @@
+// C[M,N] = f(A[M,K]) . W[N,K]^T for few rows (M <= 64): the matrix product of decode steps, where the job is to
+// stream W from HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950).
+//
+// One workgroup owns 16 rows of W (16 output columns) over the whole of K; its waves take the 32-wide steps of
+// K in turn, so together they read each weight row in contiguous runs. W rows are the A operand straight from
+// global memory (16 bytes per lane), the activations are the B operand straight from L2 (they are a few KB
+// and every workgroup reads the same ones), so no LDS is used for operands. Partial sums of the waves are
+// added through LDS in a fixed order: a row's result does not depend on M or on the other rows.
+//
+// Fused around the product, so that a layer needs fewer launches and no round trips for small tensors:
+//   NORM      the reference's RMSNorm of the input rows (main_models_new.py:38-42): the activations are multiplied
+//             by the gain on the way in, their squares are summed as they pass, and the row factor
+//             sqrt(K) / (||x|| + eps) is applied to the 32-bit sums at the end (the factor is per row, so it
+//             commutes with the product)
+//   RESIDUAL  C += R
+//   SWIGLU    W holds gate and up rows interleaved (gate_0, up_0, gate_1, ...): out[:, f] = silu(c[2f]) * c[2f+1]
+//             (main_models_new.py:51), written [M, N/2]
+// Output bfloat16 or float (the output table writes 32-bit logits).
+#include "common.h"
+
+TIS_DEFINE_LAST_ERROR(tis_gemm_skinny)
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+
+enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+
+// GS_WAVES: waves per workgroup. Sixteen where K is long enough to give each of them work: then nearly all of a
+// matrix of a few MB is requested from HBM at once and the kernel takes about one memory round trip.
+template <int MB, bool NORM, int EPI, typename TO, int GS_WAVES>
+__global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
+    const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const float* __restrict__ gain, float eps,
+    const bf16* __restrict__ R, long r_ld, TO* __restrict__ C, long c_ld, int M, int N, int K) {
+  __shared__ float red[GS_WAVES][MB][64][4];
+  __shared__ float red_ss[GS_WAVES][MB][16];
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int steps = (K + 31) / 32;
+  const bool w_ok = n0 + c16 < N;
+  const bf16* wrow = W + (long)(n0 + c16) * K + g * 8;
+
+  f32x4 acc[MB];
+  float ss[MB];
+  const bf16* xrow[MB];
+  bool x_ok[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    acc[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    ss[mb] = 0.f;
+    const int m = mb * 16 + c16;
+    x_ok[mb] = m < M;
+    xrow[mb] = X + (long)(x_ok[mb] ? m : 0) * x_ld + g * 8;
+  }
+
+  // four steps at a time: all their loads are issued before the first product, so that a wave keeps several
+  // rows' worth of HBM requests in flight
+  constexpr int U = 4;
+  for (int s0 = wave; s0 < steps; s0 += U * GS_WAVES) {
+    bf16x8 a[U];
+    bf16x8 b[U][MB];
+    float gv[U][8];
+    bool k_ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * GS_WAVES;
+      const int k = s * 32 + g * 8;
+      k_ok[u] = s < steps && k < K;   // K is a multiple of 8, so a lane's 8 values are all inside or all outside
+      a[u] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+      if (w_ok && k_ok[u]) a[u] = *reinterpret_cast<const bf16x8*>(wrow + (long)s * 32);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        b[u][mb] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+        if (x_ok[mb] && k_ok[u]) b[u][mb] = *reinterpret_cast<const bf16x8*>(xrow[mb] + (long)s * 32);
+      }
+      if (NORM) {
+        const float4 g0 = k_ok[u] ? *reinterpret_cast<const float4*>(gain + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 g1 = k_ok[u] ? *reinterpret_cast<const float4*>(gain + k + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        gv[u][0] = g0.x; gv[u][1] = g0.y; gv[u][2] = g0.z; gv[u][3] = g0.w;
+        gv[u][4] = g1.x; gv[u][5] = g1.y; gv[u][6] = g1.z; gv[u][7] = g1.w;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        bf16x8 bv = b[u][mb];
+        if (NORM) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float xf = static_cast<float>(bv[e]);
+            ss[mb] += xf * xf;
+            bv[e] = static_cast<__bf16>(xf * gv[u][e]);
+          }
+        }
+        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc[mb], 0, 0, 0);
+      }
+    }
+  }
+
+  // add the waves' partial sums in a fixed order
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][mb][lane][i] = acc[mb][i];
+    if (NORM) {
+      float t = ss[mb];
+      t += __shfl_xor(t, 16, 64);
+      t += __shfl_xor(t, 32, 64);
+      if (g == 0) red_ss[wave][mb][c16] = t;
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int m = mb * 16 + c16;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float t = red[0][mb][lane][i];
+#pragma unroll
+      for (int w = 1; w < GS_WAVES; ++w) t += red[w][mb][lane][i];
+      v[i] = t;
+    }
+    if (NORM) {
+      float t = red_ss[0][mb][c16];
+#pragma unroll
+      for (int w = 1; w < GS_WAVES; ++w) t += red_ss[w][mb][c16];
+      const float mul = sqrtf((float)K) / (sqrtf(t) + eps);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= mul;
+    }
+    if (m >= M) continue;
+    const int n = n0 + g * 4;   // the lane's four consecutive output columns
+    if (EPI == EPI_SWIGLU) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (n + 2 * j + 1 < N) {
+          const float gt = v[2 * j], up = v[2 * j + 1];
+          C[(long)m * c_ld + n / 2 + j] = from_f<TO>(gt / (1.f + __expf(-gt)) * up);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (n + i < N) {
+          float t = v[i];
+          if (EPI == EPI_RESIDUAL) t += static_cast<float>(R[(long)m * r_ld + n + i]);
+          C[(long)m * c_ld + n + i] = from_f<TO>(t);
+        }
+      }
+    }
+  }
+}
+
+template <int MB, bool NORM, int EPI, typename TO>
+static void launch(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
+                   void* C, long c_ld, int M, int N, int K, hipStream_t stream) {
+  if ((K + 31) / 32 >= 32)
+    gemm_skinny_kernel<MB, NORM, EPI, TO, 16><<<(N + 15) / 16, 16 * 64, 0, stream>>>(
+        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K);
+  else
+    gemm_skinny_kernel<MB, NORM, EPI, TO, 4><<<(N + 15) / 16, 4 * 64, 0, stream>>>(
+        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K);
+}
+
+template <bool NORM, int EPI, typename TO>
+static int launch_mb(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
+                     void* C, long c_ld, int M, int N, int K, hipStream_t stream) {
+  if (M <= 16) launch<1, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream);
+  else if (M <= 32) launch<2, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream);
+  else launch<4, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream);
+  return tis_launch_status("gemm_skinny");
+}
+
+// epilogue: 0 none, 1 residual, 2 swiglu. out_dtype: 0 float, 1 bfloat16. gain == null: no norm.
+TIS_EXPORT int tis_gemm_skinny(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R,
+                               long r_ld, void* C, long c_ld, int M, int N, int K, int epilogue, int out_dtype,
+                               hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  if (M < 0 || M > 64) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..64", M);
+  if (N < 1 || K < 8 || K % 8) return tis_fail("gemm_skinny: N=%d K=%d; K must be a multiple of 8", N, K);
+  if (x_ld % 8 || ((uintptr_t)X % 16) || ((uintptr_t)W % 16))
+    return tis_fail("gemm_skinny: activations and weights must be 16-byte aligned with row strides in steps of 8");
+  if (epilogue == EPI_RESIDUAL && !R) return tis_fail("gemm_skinny: residual epilogue without a residual");
+  if (epilogue == EPI_SWIGLU && (N % 2)) return tis_fail("gemm_skinny: gate/up rows come in pairs, N=%d is odd", N);
+  const bool norm = gain != nullptr;
+#define GO(NORMV, EPIV, TOV) return launch_mb<NORMV, EPIV, TOV>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream)
+  if (out_dtype == TIS_BF16) {
+    if (epilogue == EPI_NONE) { if (norm) GO(true, EPI_NONE, bf16); else GO(false, EPI_NONE, bf16); }
+    if (epilogue == EPI_RESIDUAL) { if (norm) GO(true, EPI_RESIDUAL, bf16); else GO(false, EPI_RESIDUAL, bf16); }
+    if (epilogue == EPI_SWIGLU) { if (norm) GO(true, EPI_SWIGLU, bf16); else GO(false, EPI_SWIGLU, bf16); }
+  } else if (out_dtype == TIS_F32) {
+    if (epilogue == EPI_NONE) { if (norm) GO(true, EPI_NONE, float); else GO(false, EPI_NONE, float); }
+  }
+#undef GO
+  return tis_fail("gemm_skinny: unsupported epilogue %d with output dtype %d", epilogue, out_dtype);
+}

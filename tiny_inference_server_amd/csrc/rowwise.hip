@@ -67,14 +67,14 @@ __global__ __launch_bounds__(ROW_THREADS) void copy_rows_kernel(const T* src, lo
   for (int c = threadIdx.x; c < D; c += blockDim.x) to[c] = from[c];
 }
 
-// out[r, f] = silu(gu[r, f]) * gu[r, F + f]      (reference main_models_new.py:51)
+// out[r, f] = silu(gu[r, 2f]) * gu[r, 2f + 1]: gate and up columns come interleaved  (reference main_models_new.py:51)
 template <typename T>
 __global__ __launch_bounds__(ROW_THREADS) void swiglu_kernel(const T* gu, long gu_ld, T* out, long out_ld, int F) {
   const long r = blockIdx.x;
   const int f = blockIdx.y * blockDim.x + threadIdx.x;
   if (f >= F) return;
-  const float g = to_f(gu[r * gu_ld + f]);
-  const float u = to_f(gu[r * gu_ld + F + f]);
+  const float g = to_f(gu[r * gu_ld + 2 * f]);
+  const float u = to_f(gu[r * gu_ld + 2 * f + 1]);
   out[r * out_ld + f] = from_f<T>(g / (1.f + expf(-g)) * u);
 }
 

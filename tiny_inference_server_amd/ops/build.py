@@ -36,7 +36,7 @@ SOURCES: Dict[str, str] = {
     "attention_generic": "attention_generic.hip",
     "attention_mfma": "attention_mfma.hip",
     "gemm_plain": "gemm_plain.hip",
-    "gemm_bf16": "gemm_bf16.hip",
+    "gemm_skinny": "gemm_skinny.hip",
     "sampling": "sampling.hip",
 }
 HEADERS = ["common.h"]

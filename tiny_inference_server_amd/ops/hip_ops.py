@@ -74,6 +74,9 @@ _SIGNATURES = {
     }),
 }
 
+_SIGNATURES["gemm_skinny"] = ("tis_gemm_skinny", {
+    "tis_gemm_skinny": [_P, _L, _P, _P, _F, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P],
+})
 _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
     "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
 })
@@ -91,7 +94,8 @@ def library(name: str) -> _Lib:
 
 
 # wavefronts the attention launch aims for, so that short batches still spread over the chip
-_ATTN_TARGET_WAVES = 1024
+_ATTN_TARGET_WAVES = 512
+_ATTN_MIN_SPLIT_KEYS = 128      # a split shorter than this costs more in merging than it gains in spreading
 _ATTN_WORKSPACE_FLOATS = 16 << 20
 
 
@@ -133,12 +137,14 @@ class HipOps:
         self.dtype = dtype
         self.code = _DT[dtype]
         # whatever is not built yet is compiled side by side, not one after the other
-        _build.build(["rowwise", "rope_cache", "attention_generic", "gemm_plain", "sampling"])
+        _build.build(["rowwise", "rope_cache", "attention_generic", "gemm_plain", "sampling"] +
+                     (["gemm_skinny"] if dtype == torch.bfloat16 else []))
         self.rowwise = library("rowwise")
         self.rope = library("rope_cache")
         self.attn_generic = library("attention_generic")
         self.gemm_plain = library("gemm_plain")
         self.sampling = library("sampling")
+        self.gemm_skinny = library("gemm_skinny") if dtype == torch.bfloat16 else None
         self._attn_groups = set()          # group sizes of the attention mixers built on these ops
         self._attn_mfma = {}               # head size -> library
         self._workspace = None
@@ -259,7 +265,7 @@ class HipOps:
                                    _ptr(dst_index), n, src.shape[1], self._stream())
 
     def swiglu(self, gu, out=None):
-        """out[:, f] = silu(gu[:, f]) * gu[:, F + f]."""
+        """out[:, f] = silu(gu[:, 2f]) * gu[:, 2f + 1]: gate and up columns interleaved."""
         _rows_view(self._check(gu, "swiglu in"), "swiglu in")
         n, F2 = gu.shape
         if F2 % 2:
@@ -274,8 +280,11 @@ class HipOps:
         return out
 
     # ---- matrix products -----------------------------------------------------------------------------
-    def linear(self, x, w, residual=None, out_dtype=None):
-        """x[M,K] . w[N,K]^T (+ residual[M,N]); `out_dtype` float32 gives 32-bit results from bfloat16 inputs."""
+    def linear(self, x, w, residual=None, out_dtype=None, rms=None):
+        """f(x)[M,K] . w[N,K]^T (+ residual[M,N]); `out_dtype` float32 gives 32-bit results from bfloat16 inputs.
+
+        rms = (gain, eps): f is the RMSNorm of the rows, fused into the product where the kernel allows.
+        """
         _rows_view(self._check(x, "linear x"), "linear x")
         self._check(w, "linear w")
         out_dtype = out_dtype or self.dtype
@@ -287,6 +296,19 @@ class HipOps:
             _rows_view(self._check(residual, "linear residual", out_dtype), "linear residual")
             if tuple(residual.shape) != (M, N):
                 raise KernelError(f"linear: residual {tuple(residual.shape)} for result {(M, N)}")
+        if rms is not None:
+            self._check(rms[0], "rmsnorm gain", torch.float32)
+            if rms[0].numel() != K or not rms[0].is_contiguous():
+                raise KernelError(f"linear: norm gain has {rms[0].numel()} entries for width {K}")
+        if self._skinny_ok(x, M, K):
+            out = self.empty(M, N, dtype=out_dtype)
+            self.gemm_skinny.tis_gemm_skinny(
+                _ptr(x), x.stride(0), _ptr(w), _ptr(rms[0] if rms else None), float(rms[1]) if rms else 0.0,
+                _ptr(residual), residual.stride(0) if residual is not None else 0, _ptr(out), N, M, N, K,
+                1 if residual is not None else 0, _DT[out_dtype], self._stream())
+            return out
+        if rms is not None:
+            x = self.rmsnorm(x, rms[0], rms[1])
         if self.dtype == torch.float32:
             out = self.empty(M, N, dtype=torch.float32)
             self.gemm_plain.tis_gemm_plain(0, 0, _ptr(x), x.stride(0), _ptr(w), K, _ptr(residual),
@@ -294,6 +316,28 @@ class HipOps:
                                            self._stream())
             return out
         return self._linear_bf16(x, w, residual, out_dtype)
+
+    def _skinny_ok(self, x, M, K):
+        return (self.dtype == torch.bfloat16 and 0 < M <= 64 and K % 8 == 0 and x.stride(0) % 8 == 0
+                and x.data_ptr() % 16 == 0)
+
+    def linear_swiglu(self, x, w, rms=None):
+        """silu(g) * u of the rows of f(x) . w^T, w holding gate and up rows interleaved: [M, N/2]."""
+        _rows_view(self._check(x, "linear x"), "linear x")
+        M, K = x.shape
+        if self._skinny_ok(x, M, K) and w.shape[0] % 2 == 0:
+            self._check(w, "linear w")
+            if w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+                raise KernelError(f"linear: x {tuple(x.shape)} against w {tuple(w.shape)} (w is [out, in], contiguous)")
+            if rms is not None and (rms[0].numel() != K or rms[0].dtype != torch.float32):
+                raise KernelError(f"linear: norm gain has {rms[0].numel()} entries for width {K}")
+            N = w.shape[0]
+            out = self.empty(M, N // 2)
+            self.gemm_skinny.tis_gemm_skinny(
+                _ptr(x), x.stride(0), _ptr(w), _ptr(rms[0] if rms else None), float(rms[1]) if rms else 0.0,
+                _ptr(None), 0, _ptr(out), N // 2, M, N, K, 2, 1, self._stream())
+            return out
+        return self.swiglu(self.linear(x, w, rms=rms))
 
     def _linear_bf16(self, x, w, residual, out_dtype):
         if out_dtype == torch.float32:
@@ -370,7 +414,8 @@ class HipOps:
             lib = self._attn_mfma.get(head_dim)
             if lib is None:
                 lib = self._attn_mfma[head_dim] = library(f"attention_mfma@{head_dim}")
-            n_splits = max(1, min(-(-_ATTN_TARGET_WAVES // (n_items * n_kv_heads)), -(-batch.max_kv_len // 64)))
+            n_splits = max(1, min(-(-_ATTN_TARGET_WAVES // (n_items * n_kv_heads)),
+                                  batch.max_kv_len // _ATTN_MIN_SPLIT_KEYS))
             # partial results of split key ranges live in one workspace of fixed size, allocated once and never
             # moved (captured graphs hold its address); fewer splits where it would not suffice
             n_splits = max(1, min(n_splits, _ATTN_WORKSPACE_FLOATS // (n * n_heads * (head_dim + 2))))

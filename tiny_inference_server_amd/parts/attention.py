@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import MIXERS, build_part, to_compute
+from .base import MIXERS, build_part, normed_linear, to_compute
 from .spec import PagedKvNeed
 
 
@@ -48,9 +48,11 @@ class GqaAttention:
         if hasattr(ops, "register_attention"):
             ops.register_attention(self.n_heads, self.n_kv_heads, self.head_dim)
 
-    def forward(self, x, ctx, residual=None):
+    fuses_norm = True
+
+    def forward(self, x, ctx, residual=None, norm=None):
         ops, b = self.ops, ctx.batch
-        qkv = ops.linear(x, self.w_qkv)
+        qkv = normed_linear(ops, x, self.w_qkv, norm)
         table, interleaved = self.position.rotary()
         page_size = ctx.plane.shape[3]
         ops.rope_write_kv(qkv, b.positions, b.write_slots[ctx.group], table, ctx.plane, self.n_heads,

@@ -20,6 +20,9 @@ every part      graph_safe = True                      class attribute, only if 
 mixer           cache_need(params) -> PagedKvNeed | StateNeed | None      classmethod
                 forward(x, ctx, residual=None) -> y    x: normed rows; ctx: CallContext; adds `residual` if given
 feed-forward    forward(x, residual=None) -> y
+                a mixer or feed-forward with the class attribute fuses_norm = True takes forward(..., norm=part)
+                instead: x arrives un-normed and the part applies `norm` itself, fused into its first product
+                where it can
 arrangement     __init__(layer_spec, parts...), forward(x, ctx) -> x      how norm, mixer and feed-forward are wired
 stage input     state_need(params) -> StateNeed | None classmethod
                 forward(batch, previous_output, previous_batch, shared, state) -> rows
@@ -91,6 +94,15 @@ def expected_tensors(spec):
         if hasattr(v, "role") and hasattr(v, "kind"):
             out.update(expected_tensors(v))
     return out
+
+
+def normed_linear(ops, x, w, norm, **kw):
+    """norm(x) . w^T: through the fused kernel if the norm offers its (gain, eps), else in two steps."""
+    if norm is None:
+        return ops.linear(x, w, **kw)
+    if hasattr(norm, "as_rms"):
+        return ops.linear(x, w, rms=norm.as_rms(), **kw)
+    return ops.linear(norm(x), w, **kw)
 
 
 def to_compute(ops, t):

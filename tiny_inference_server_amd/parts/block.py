@@ -15,5 +15,10 @@ class PreNormResidual:
         self.ffn = build_part(layer_spec.feed_forward, tensors, ops)
 
     def forward(self, x, ctx):
-        x = self.mixer.forward(self.mixer_norm(x), ctx, residual=x)
+        if getattr(self.mixer, "fuses_norm", False):
+            x = self.mixer.forward(x, ctx, residual=x, norm=self.mixer_norm)
+        else:
+            x = self.mixer.forward(self.mixer_norm(x), ctx, residual=x)
+        if getattr(self.ffn, "fuses_norm", False):
+            return self.ffn.forward(x, residual=x, norm=self.ffn_norm)
         return self.ffn.forward(self.ffn_norm(x), residual=x)

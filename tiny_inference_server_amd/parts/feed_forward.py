@@ -22,10 +22,17 @@ class SwiGlu:
 
     def __init__(self, spec, tensors, ops):
         self.ops = ops
-        # one projection for gate and up: rows [0, hidden) of the [out, in] matrix are the gate
-        self.w_gate_up = to_compute(ops, torch.cat((tensors.of(spec, "gate"), tensors.of(spec, "up")), dim=1).t())
+        # one projection for gate and up: rows of the [out, in] matrix alternate gate_0, up_0, gate_1, up_1, ...
+        # so that the gating can be done where the product's results still sit in registers
+        gate, up = tensors.of(spec, "gate"), tensors.of(spec, "up")
+        self.w_gate_up = to_compute(ops, torch.stack((gate.t(), up.t()), dim=1).reshape(2 * gate.shape[1], gate.shape[0]))
         self.w_down = to_compute(ops, tensors.of(spec, "down").t())
 
-    def forward(self, x, residual=None):
+    fuses_norm = True
+
+    def forward(self, x, residual=None, norm=None):
         ops = self.ops
-        return ops.linear(ops.swiglu(ops.linear(x, self.w_gate_up)), self.w_down, residual=residual)
+        if norm is not None and not hasattr(norm, "as_rms"):
+            x, norm = norm(x), None
+        hidden = ops.linear_swiglu(x, self.w_gate_up, rms=norm.as_rms() if norm is not None else None)
+        return ops.linear(hidden, self.w_down, residual=residual)

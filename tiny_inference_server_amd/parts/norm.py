@@ -23,5 +23,9 @@ class RmsNormL2:
         self.eps = float(spec.params["eps"])
         self.gain = to_gain(ops, tensors.of(spec, "gain"))
 
+    def as_rms(self):
+        """(gain, eps) for kernels that fuse this norm into what follows it."""
+        return self.gain, self.eps
+
     def __call__(self, x, out=None):
         return self.ops.rmsnorm(x, self.gain, self.eps, out=out)

@@ -109,11 +109,16 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     bf16x8 v[DB];
     bool ok[2];
   };
+  // Every load below is unconditional: a tile that lies past the item's keys, or a step past the wave's share,
+  // reads page 0 instead (always mapped, and finite) and is masked afterwards. Without branches around the loads
+  // the compiler can wait for exactly the loads a product needs while the next step's are still in flight.
   auto page_ids = [&](int s, int (&pg)[2]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int key0 = k_lo + s * 32 + t * 16;
-      pg[t] = (s < s_end && key0 < k_hi) ? bt[key0 / page_size] : -1;
+      const bool ok = s < s_end && key0 < k_hi;
+      const int got = bt[ok ? key0 / page_size : 0];
+      pg[t] = ok ? got : -1;
     }
   };
   auto load_tiles = [&](int s, const int (&pg)[2], Tiles& T) {
@@ -123,18 +128,18 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
       const int slot0 = key0 % page_size;
       T.ok[t] = pg[t] >= 0;
       const bf16* base = plane + (long)(T.ok[t] ? pg[t] : 0) * page_stride;
-      const bf16* kp = base + k_head + (long)(slot0 + c16) * HD + g * 8;
+      const bf16* kp = base + k_head + (long)(slot0 + c16) * HD;
       const bf16* vp = base + v_head + (long)c16 * page_size + slot0 + g * 4;
 #pragma unroll
       for (int dc = 0; dc < DC; ++dc) {
-        bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (T.ok[t] && dc * 32 + g * 8 < HD) ka = load8(kp + dc * 32);
-        T.k[t][dc] = ka;
+        const int d = dc * 32 + g * 8;
+        const bool d_ok = (HD % 32 == 0) || d < HD;
+        const bf16x8 ka = load8(kp + (d_ok ? d : 0));
+        T.k[t][dc] = d_ok ? ka : (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
       }
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        bf16x4 h = {0, 0, 0, 0};
-        if (T.ok[t]) h = load4(vp + (long)db * 16 * page_size);
+        const bf16x4 h = load4(vp + (long)db * 16 * page_size);
 #pragma unroll
         for (int e = 0; e < 4; ++e) T.v[db][t * 4 + e] = h[e];
       }
@@ -202,21 +207,18 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
 
   if (s_begin < s_end) {
     Tiles ta, tb;
-    int pa[2], pn[2];
+    int pa[2], pn[2], pq[2];
     page_ids(s_begin, pa);
     page_ids(s_begin + 1, pn);
     load_tiles(s_begin, pa, ta);
     for (int s = s_begin; s < s_end; s += 2) {
-      // pn holds the page ids of step s+1
-      int pq[2];
+      // pn holds the page ids of step s+1; loads past the end are harmless and never consumed
       page_ids(s + 2, pq);
-      if (s + 1 < s_end) load_tiles(s + 1, pn, tb);
+      load_tiles(s + 1, pn, tb);
       consume(s, ta);
-      if (s + 1 < s_end) {
-        page_ids(s + 3, pn);
-        if (s + 2 < s_end) load_tiles(s + 2, pq, ta);
-        consume(s + 1, tb);
-      }
+      page_ids(s + 3, pn);
+      load_tiles(s + 2, pq, ta);
+      if (s + 1 < s_end) consume(s + 1, tb);
     }
   }
 

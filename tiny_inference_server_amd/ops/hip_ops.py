@@ -111,10 +111,13 @@ def attention_items(seq_rows, group_size: int):
         nb *= 2
     per_item = max(1, (16 * nb) // group_size)
     items = []
-    for first, _, n in seq_rows:
+    for first, p0, n in seq_rows:
         for r in range(0, n, per_item):
-            items.append((first + r, min(per_item, n - r)))
-    return nb, items
+            items.append((p0 + r + min(per_item, n - r), first + r, min(per_item, n - r)))
+    # the items with the most keys first: under a causal mask the last rows of a prompt are the longest, and
+    # started last they would run on alone while the rest of the chip idles
+    items.sort(key=lambda it: -it[0])
+    return nb, [(first, n) for _, first, n in items]
 
 
 def _rows_view(t: torch.Tensor, what: str):

@@ -292,3 +292,69 @@ def test_sampling_reference_vectors(ops_for):
     args = (one(1.0), one(1, torch.int32), one(0.0))
     assert ops.sample(lg.cuda(), *args, one(1.0), one(0.5)).item() == 5
     assert ops.sample(lg.cuda(), *args, one(2.0), one(0.5), one(5, torch.int32), torch.tensor([0, 1], dtype=torch.int32).cuda()).item() == 7
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(96, 64), (1000, 96), (130, 264), (2304, 1536), (1536, 4096)])
+def test_skinny_product_with_fused_norm_residual_and_gate(ops_for, M, N, K):
+    """The few-row matrix-core product and what is fused around it, against the unfused plain computation."""
+    ops, ref = ops_for(torch.bfloat16), TorchOps(dtype=torch.bfloat16)
+    x, w, res = rnd((M, K), torch.bfloat16, 80, 2.0), rnd((N, K), torch.bfloat16, 81, K ** -0.5), rnd((M, N), torch.bfloat16, 82)
+    gain = 1 + 0.1 * rnd((K,), torch.float32, 83)
+    # the kernel's own rounding points, then exact arithmetic: the activations times the gain are rounded to
+    # bfloat16, the row factor sqrt(K)/(||x||+eps) multiplies the 32-bit sums. Only the output's rounding is left,
+    # so the comparison is tight (half a unit of bfloat16 is 0.4 % of a value).
+    t = dict(rtol=8e-3, atol=2e-3)
+    xb = (x.float() * gain).to(torch.bfloat16).double()
+    mul = (K ** 0.5) / (x.double().norm(dim=-1, keepdim=True) + 1e-5)
+    normed = (xb @ w.double().t()) * mul
+    torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), normed, **t)
+    # and that is the reference's norm followed by the product, up to bfloat16 rounding of the normed rows
+    xn = ref.rmsnorm(x, gain, 1e-5).double()
+    assert ((xn @ w.double().t()) - normed).abs().max() < 0.05
+    torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), residual=res.cuda()).cpu().double(),
+                               x.double() @ w.double().t() + res.double(), **t)
+    lg = ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32)
+    assert lg.dtype == torch.float32
+    torch.testing.assert_close(lg.cpu().double(), x.double() @ w.double().t(), rtol=1e-4, atol=1e-4)   # 32-bit sums kept
+    want = torch.nn.functional.silu(normed[:, 0::2]) * normed[:, 1::2]
+    torch.testing.assert_close(ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), want, **t)
+    # a row's result does not depend on the other rows of the batch
+    alone = ops.linear(x[:1].cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()
+    assert torch.equal(alone[0], ops.linear(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()[0])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M", [1, 5, 64, 200])
+@pytest.mark.parametrize("n_heads,n_kv,hd,page_size,interleaved", [(8, 2, 8, 16, False), (3, 1, 32, 8, False),
+                                                                    (12, 3, 128, 16, False), (4, 2, 48, 16, True)])
+def test_projection_with_rotary_and_cache_write(ops_for, dtype, M, n_heads, n_kv, hd, page_size, interleaved):
+    """q/k/v projection + rotary + cache write: one kernel for few bfloat16 rows, two otherwise; same results."""
+    ops, ref = ops_for(dtype), TorchOps(dtype=dtype)
+    K, n_pages, max_ctx = 96, -(-M // page_size) + 3, 300
+    N = (n_heads + 2 * n_kv) * hd
+    j = torch.arange(hd // 2)
+    ang = torch.outer(torch.arange(max_ctx).float(), 1.0 / torch.pow(torch.tensor(1e4), (2 * j.float()) / hd))
+    table = torch.stack((torch.cos(ang), torch.sin(ang)), -1).contiguous()
+    x, w = rnd((M, K), dtype, 84), rnd((N, K), dtype, 85, K ** -0.5)
+    gain = 1 + 0.1 * rnd((K,), torch.float32, 86)
+    positions = torch.tensor(random.Random(87).choices(range(max_ctx), k=M), dtype=torch.int32)
+    slots = torch.tensor(random.Random(88).sample(range(n_pages * page_size), M), dtype=torch.int32)
+    plane0 = rnd((n_pages, 2, n_kv, page_size, hd), dtype, 89)
+    pa, pb = plane0.clone().cuda(), plane0.clone()
+    got = ops.qkv_rope(x.cuda(), w.cuda(), (gain.cuda(), 1e-5), positions.cuda(), slots.cuda(), table.cuda(), pa, n_heads,
+                       n_kv, hd, page_size, interleaved).cpu()
+    want = ref.qkv_rope(x, w, (gain, 1e-5), positions, slots, table, pb, n_heads, n_kv, hd, page_size, interleaved)
+    t = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+    torch.testing.assert_close(got.float(), want.float(), **t)
+    torch.testing.assert_close(pa.cpu().float(), pb.float(), **t)
+    # against the formula itself: natural-order weights, rotate_half pairing (reference main_models_new.py:71-80)
+    if not interleaved:
+        half = hd // 2
+        order = torch.stack((torch.arange(half), torch.arange(half) + half), dim=1).reshape(-1)
+        inv = torch.argsort(order)
+        wq = w[:n_heads * hd].view(n_heads, hd, K)[:, inv].reshape(n_heads * hd, K)      # back to natural order
+        q = (ref.rmsnorm(x, gain, 1e-5).double() @ wq.double().t()).view(M, n_heads, hd)
+        c, s = table[positions.long()][..., 0].double().repeat(1, 2).unsqueeze(1), table[positions.long()][..., 1].double().repeat(1, 2).unsqueeze(1)
+        rot = torch.cat((-q[..., half:], q[..., :half]), dim=-1)
+        torch.testing.assert_close(got.double().view(M, n_heads, hd), q * c + rot * s, **t)

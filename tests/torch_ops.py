@@ -72,12 +72,27 @@ class TorchOps:
         return self.swiglu(self.linear(x, w, rms=rms))
 
     # ---- rotary + cache write ---------------------------------------------------------------------------
+    def qkv_rope(self, x, w, rms, positions, write_slots, table, plane, n_heads, n_kv_heads, head_dim, page_size,
+                 interleaved=False, write_cache=True):
+        qkv = self.linear(x, w, rms=rms)
+        q = torch.zeros(x.shape[0], n_heads * head_dim, dtype=qkv.dtype, device=qkv.device)
+        self.rope_write_kv(qkv, positions, write_slots, table, plane, n_heads, n_kv_heads, head_dim, page_size,
+                           interleaved, write_cache, paired=True, q_out=q)
+        return q
+
     def rope_write_kv(self, qkv, positions, write_slots, table, plane, n_heads, n_kv_heads, head_dim, page_size,
-                      interleaved=False, write_cache=True):
+                      interleaved=False, write_cache=True, paired=False, q_out=None):
         n = qkv.shape[0]
         if n == 0:
             return
+        qkv = qkv if not paired else qkv.clone()
         x = qkv.view(n, n_heads + 2 * n_kv_heads, head_dim)
+        if paired:
+            # pair j sits at columns 2j, 2j+1 of every q and k head: put the heads back in natural order first
+            qk_p = x[:, :n_heads + n_kv_heads]
+            first, second = qk_p[..., 0::2], qk_p[..., 1::2]
+            nat = torch.stack((first, second), dim=-1).flatten(-2) if interleaved else torch.cat((first, second), dim=-1)
+            x[:, :n_heads + n_kv_heads] = nat
         qk = x[:, :n_heads + n_kv_heads].float()
         if table is not None:
             cs = table[positions.long()]                     # [n, hd/2, 2]
@@ -90,6 +105,8 @@ class TorchOps:
                 a, b = qk[..., :h], qk[..., h:]
                 rot = torch.cat((a * c - b * s, b * c + a * s), dim=-1)
             x[:, :n_heads + n_kv_heads] = rot.to(qkv.dtype)
+        if q_out is not None:
+            q_out.copy_(x[:, :n_heads].reshape(n, n_heads * head_dim))
         if write_cache:
             slots = write_slots.long()
             page, off = slots // page_size, slots % page_size

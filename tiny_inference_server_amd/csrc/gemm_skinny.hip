@@ -25,14 +25,27 @@ typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 
-enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
+
+// What the rotary epilogue needs beyond the product: the rows of W are [q heads | k heads | v heads], and inside
+// every q and k head the rows are ordered so that the two members of a rotary pair are neighbours
+// (pair j at rows 2j and 2j+1). The epilogue rotates each pair by the row's position, puts queries back in
+// their natural order into `C` ([M, n_heads*head_dim]) and writes keys and values into the cache page of the
+// row's slot: keys as [slot][head_dim], values transposed as [head_dim][slot].
+struct RopeArgs {
+  const int* positions;
+  const int* write_slots;
+  const float2* table;     // [position][pair] (cos, sin); null: no rotation
+  bf16* plane;
+  int n_heads, n_kv_heads, head_dim, page_size, interleaved, write_cache;
+};
 
 // GS_WAVES: waves per workgroup. Sixteen where K is long enough to give each of them work: then nearly all of a
 // matrix of a few MB is requested from HBM at once and the kernel takes about one memory round trip.
 template <int MB, bool NORM, int EPI, typename TO, int GS_WAVES>
 __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
     const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const float* __restrict__ gain, float eps,
-    const bf16* __restrict__ R, long r_ld, TO* __restrict__ C, long c_ld, int M, int N, int K) {
+    const bf16* __restrict__ R, long r_ld, TO* __restrict__ C, long c_ld, int M, int N, int K, RopeArgs rope) {
   __shared__ float red[GS_WAVES][MB][64][4];
   __shared__ float red_ss[GS_WAVES][MB][16];
 
@@ -136,7 +149,45 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
     }
     if (m >= M) continue;
     const int n = n0 + g * 4;   // the lane's four consecutive output columns
-    if (EPI == EPI_SWIGLU) {
+    if (EPI == EPI_ROPE) {
+      if (n >= N) continue;          // N is a multiple of head_dim, head_dim of 4: the lane's columns are all in or out
+      const int hd = rope.head_dim, half = hd / 2;
+      const int head = n / hd, e0 = n % hd;      // e0 is a multiple of 4: two whole pairs
+      const bool is_q = head < rope.n_heads, is_v = head >= rope.n_heads + rope.n_kv_heads;
+      float y[4] = {v[0], v[1], v[2], v[3]};
+      int d[4];                                   // where the lane's four values belong inside the head
+      if (is_v) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) d[i] = e0 + i;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int pair = e0 / 2 + j;
+          d[2 * j] = rope.interleaved ? 2 * pair : pair;
+          d[2 * j + 1] = rope.interleaved ? 2 * pair + 1 : pair + half;
+          if (rope.table) {
+            const float2 cs = rope.table[(long)rope.positions[m] * half + pair];
+            const float x1 = v[2 * j], x2 = v[2 * j + 1];
+            y[2 * j] = x1 * cs.x - x2 * cs.y;
+            y[2 * j + 1] = x2 * cs.x + x1 * cs.y;
+          }
+        }
+      }
+      if (is_q) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) C[(long)m * c_ld + (long)head * hd + d[i]] = from_f<TO>(y[i]);
+      } else if (rope.write_cache) {
+        const int slot = rope.write_slots[m];
+        const int page = slot / rope.page_size, off = slot % rope.page_size;
+        const int kvh = is_v ? head - rope.n_heads - rope.n_kv_heads : head - rope.n_heads;
+        bf16* hp = rope.plane + (((long)page * 2 + (is_v ? 1 : 0)) * rope.n_kv_heads + kvh) * rope.page_size * hd;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (is_v) hp[(long)d[i] * rope.page_size + off] = static_cast<__bf16>(y[i]);
+          else hp[(long)off * hd + d[i]] = static_cast<__bf16>(y[i]);
+        }
+      }
+    } else if (EPI == EPI_SWIGLU) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         if (n + 2 * j + 1 < N) {
@@ -159,21 +210,21 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
 
 template <int MB, bool NORM, int EPI, typename TO>
 static void launch(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
-                   void* C, long c_ld, int M, int N, int K, hipStream_t stream) {
+                   void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope = RopeArgs()) {
   if ((K + 31) / 32 >= 32)
     gemm_skinny_kernel<MB, NORM, EPI, TO, 16><<<(N + 15) / 16, 16 * 64, 0, stream>>>(
-        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K);
+        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);
   else
     gemm_skinny_kernel<MB, NORM, EPI, TO, 4><<<(N + 15) / 16, 4 * 64, 0, stream>>>(
-        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K);
+        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);
 }
 
 template <bool NORM, int EPI, typename TO>
 static int launch_mb(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
-                     void* C, long c_ld, int M, int N, int K, hipStream_t stream) {
-  if (M <= 16) launch<1, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream);
-  else if (M <= 32) launch<2, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream);
-  else launch<4, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream);
+                     void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope = RopeArgs()) {
+  if (M <= 16) launch<1, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
+  else if (M <= 32) launch<2, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
+  else launch<4, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
   return tis_launch_status("gemm_skinny");
 }
 
@@ -199,4 +250,34 @@ TIS_EXPORT int tis_gemm_skinny(const void* X, long x_ld, const void* W, const fl
   }
 #undef GO
   return tis_fail("gemm_skinny: unsupported epilogue %d with output dtype %d", epilogue, out_dtype);
+}
+
+// The q/k/v projection of an attention layer with the rotary encoding and the cache write in its epilogue.
+// W: [(n_heads + 2 n_kv_heads) * head_dim, K] with rotary pairs on neighbouring rows (see RopeArgs). Q out: [M, n_heads*head_dim].
+TIS_EXPORT int tis_gemm_skinny_qkv_rope(const void* X, long x_ld, const void* W, const float* gain, float eps, void* Q,
+                                        long q_ld, int M, int K, const int* positions, const int* write_slots,
+                                        const float* table, void* plane, int n_heads, int n_kv_heads, int head_dim,
+                                        int page_size, int interleaved, int write_cache, hipStream_t stream) {
+  if (M == 0) return 0;
+  if (M < 0 || M > 64) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..64", M);
+  if (K < 8 || K % 8) return tis_fail("gemm_skinny: K=%d must be a multiple of 8", K);
+  if (n_heads < 1 || n_kv_heads < 1 || head_dim < 4 || head_dim % 4 || page_size < 1)
+    return tis_fail("gemm_skinny: heads=%d kv_heads=%d head_dim=%d (a multiple of 4) page=%d", n_heads, n_kv_heads,
+                    head_dim, page_size);
+  if (x_ld % 8 || ((uintptr_t)X % 16) || ((uintptr_t)W % 16))
+    return tis_fail("gemm_skinny: activations and weights must be 16-byte aligned with row strides in steps of 8");
+  RopeArgs rope;
+  rope.positions = positions;
+  rope.write_slots = write_slots;
+  rope.table = (const float2*)table;
+  rope.plane = (bf16*)plane;
+  rope.n_heads = n_heads;
+  rope.n_kv_heads = n_kv_heads;
+  rope.head_dim = head_dim;
+  rope.page_size = page_size;
+  rope.interleaved = interleaved;
+  rope.write_cache = write_cache;
+  const int N = (n_heads + 2 * n_kv_heads) * head_dim;
+  if (gain) return launch_mb<true, EPI_ROPE, bf16>(X, x_ld, W, gain, eps, nullptr, 0, Q, q_ld, M, N, K, stream, rope);
+  return launch_mb<false, EPI_ROPE, bf16>(X, x_ld, W, gain, eps, nullptr, 0, Q, q_ld, M, N, K, stream, rope);
 }

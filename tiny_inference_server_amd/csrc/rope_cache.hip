@@ -5,6 +5,10 @@
 // (cos, sin) per position and pair. Pairs are (j, j + head_dim/2) in the "half" pairing (reference
 // main_models_new.py:71-80) or (2j, 2j+1) in the "interleaved" pairing; a null table means no rotation.
 //
+// With `paired` the q and k heads of the input come with the two members of every rotary pair side by side
+// (pair j at columns 2j and 2j+1 of the head: the order in which the fused projection's weight rows are kept);
+// the rotated queries then go, in their natural order, to a separate output.
+//
 // One cache plane is laid out [page][key or value][kv head][...]: a head's keys of a page as [slot][head_dim],
 // its values transposed as [head_dim][slot], which is how the matrix-core attention kernel wants to load them.
 #include "common.h"
@@ -16,18 +20,20 @@ __global__ __launch_bounds__(64) void rope_write_kv_kernel(T* __restrict__ qkv, 
                                                            const int* __restrict__ write_slots,
                                                            const float2* __restrict__ table, T* __restrict__ plane,
                                                            int n_heads, int n_kv_heads, int head_dim, int page_size,
-                                                           int interleaved, int write_cache) {
+                                                           int interleaved, int write_cache, int paired,
+                                                           T* __restrict__ q_out, long q_out_ld) {
   const long r = blockIdx.x;
   const int hh = blockIdx.y;  // [0, n_heads): q, then k heads, then v heads
   const int half = head_dim / 2;
   T* row = qkv + r * ld + (long)hh * head_dim;
 
-  T* dst = row;  // queries are rewritten where they are
+  T* dst = row;  // queries are rewritten where they are, unless a separate output is given
   const bool is_q = hh < n_heads;
+  if (is_q && q_out) dst = q_out + r * q_out_ld + (long)hh * head_dim;
   const bool is_v = hh >= n_heads + n_kv_heads;
   if (!is_q) {
     if (!write_cache) {
-      if (is_v) return;  // nothing to do for values
+      return;  // keys and values that are not kept have no reader
     } else {
       const int slot = write_slots[r];
       const int page = slot / page_size, off = slot % page_size;
@@ -42,15 +48,21 @@ __global__ __launch_bounds__(64) void rope_write_kv_kernel(T* __restrict__ qkv, 
   }
   if (is_v) return;
   if (table == nullptr) {
-    if (dst != row)
+    if (paired) {
+      for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        dst[interleaved ? 2 * j : j] = row[2 * j];
+        dst[interleaved ? 2 * j + 1 : j + half] = row[2 * j + 1];
+      }
+    } else if (dst != row) {
       for (int i = threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = row[i];
+    }
     return;
   }
   const float2* cs = table + (long)positions[r] * half;
   for (int j = threadIdx.x; j < half; j += blockDim.x) {
     const int a = interleaved ? 2 * j : j;
     const int b = interleaved ? 2 * j + 1 : j + half;
-    const float x1 = to_f(row[a]), x2 = to_f(row[b]);
+    const float x1 = to_f(row[paired ? 2 * j : a]), x2 = to_f(row[paired ? 2 * j + 1 : b]);
     const float c = cs[j].x, s = cs[j].y;
     // q*cos + rotate_half(q)*sin with rotate_half = [-x2, x1]
     const float y1 = x1 * c - x2 * s;
@@ -62,21 +74,23 @@ __global__ __launch_bounds__(64) void rope_write_kv_kernel(T* __restrict__ qkv, 
 
 TIS_EXPORT int tis_rope_write_kv(int dtype, void* qkv, long ld, const int* positions, const int* write_slots,
                                  const float* table, void* plane, int rows, int n_heads, int n_kv_heads, int head_dim,
-                                 int page_size, int interleaved, int write_cache, hipStream_t stream) {
+                                 int page_size, int interleaved, int write_cache, int paired, void* q_out,
+                                 long q_out_ld, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || n_heads < 1 || n_kv_heads < 1 || head_dim < 2 || (head_dim & 1) || page_size < 1)
     return tis_fail("rope_write_kv: bad size rows=%d heads=%d kv_heads=%d head_dim=%d page=%d", rows, n_heads,
                     n_kv_heads, head_dim, page_size);
   if (n_heads + 2 * n_kv_heads > 65535) return tis_fail("rope_write_kv: too many heads for the grid");
+  if (paired && !q_out) return tis_fail("rope_write_kv: paired input needs a separate output for the queries");
   dim3 grid(rows, n_heads + 2 * n_kv_heads);
   if (dtype == TIS_F32)
     rope_write_kv_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, ld, positions, write_slots, (const float2*)table,
                                                          (float*)plane, n_heads, n_kv_heads, head_dim, page_size,
-                                                         interleaved, write_cache);
+                                                         interleaved, write_cache, paired, (float*)q_out, q_out_ld);
   else if (dtype == TIS_BF16)
     rope_write_kv_kernel<bf16><<<grid, 64, 0, stream>>>((bf16*)qkv, ld, positions, write_slots, (const float2*)table,
                                                         (bf16*)plane, n_heads, n_kv_heads, head_dim, page_size,
-                                                        interleaved, write_cache);
+                                                        interleaved, write_cache, paired, (bf16*)q_out, q_out_ld);
   else
     return tis_fail("unknown dtype code %d", dtype);
   return tis_launch_status("rope_write_kv");

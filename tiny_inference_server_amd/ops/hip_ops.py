@@ -60,7 +60,7 @@ _SIGNATURES = {
         "tis_swiglu": [_I, _P, _L, _P, _L, _I, _I, _P],
     }),
     "rope_cache": ("tis_rope_cache", {
-        "tis_rope_write_kv": [_I, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+        "tis_rope_write_kv": [_I, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _L, _P],
     }),
     "attention_generic": ("tis_attention_generic", {
         "tis_attention_generic": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _F, _P],
@@ -76,6 +76,7 @@ _SIGNATURES = {
 
 _SIGNATURES["gemm_skinny"] = ("tis_gemm_skinny", {
     "tis_gemm_skinny": [_P, _L, _P, _P, _F, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P],
+    "tis_gemm_skinny_qkv_rope": [_P, _L, _P, _P, _F, _P, _L, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
 })
 _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
     "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
@@ -354,8 +355,20 @@ class HipOps:
 
     # ---- position encoding + cache write, attention --------------------------------------------------
     def rope_write_kv(self, qkv, positions, write_slots, table, plane, n_heads, n_kv_heads, head_dim, page_size,
-                      interleaved=False, write_cache=True):
+                      interleaved=False, write_cache=True, paired=False, q_out=None):
+        """Rotate q (in place, or into `q_out`) and write rotated k and v into the cache plane.
+
+        paired: the q and k heads of `qkv` hold the members of each rotary pair side by side (pair j at columns
+        2j, 2j+1), as a projection with pair-ordered weight rows leaves them; `q_out` then receives the queries
+        in natural order.
+        """
         _rows_view(self._check(qkv, "qkv"), "qkv")
+        if paired and q_out is None:
+            raise KernelError("rope_write_kv: paired input needs q_out")
+        if q_out is not None:
+            _rows_view(self._check(q_out, "q_out"), "q_out")
+            if tuple(q_out.shape) != (qkv.shape[0], n_heads * head_dim):
+                raise KernelError(f"rope_write_kv: q_out {tuple(q_out.shape)} for {qkv.shape[0]} rows of {n_heads * head_dim}")
         n = qkv.shape[0]
         if qkv.shape[1] != (n_heads + 2 * n_kv_heads) * head_dim:
             raise KernelError(f"rope_write_kv: row width {qkv.shape[1]} is not (heads {n_heads} + 2 x kv heads "
@@ -371,7 +384,45 @@ class HipOps:
         self.rope.tis_rope_write_kv(self.code, _ptr(qkv), qkv.stride(0), _ptr(positions),
                                     _ptr(write_slots if write_cache else None), _ptr(table),
                                     _ptr(plane if write_cache else None), n, n_heads, n_kv_heads, head_dim, page_size,
-                                    int(bool(interleaved)), int(bool(write_cache)), self._stream())
+                                    int(bool(interleaved)), int(bool(write_cache)), int(bool(paired)), _ptr(q_out),
+                                    q_out.stride(0) if q_out is not None else 0, self._stream())
+
+    def qkv_rope(self, x, w, rms, positions, write_slots, table, plane, n_heads, n_kv_heads, head_dim, page_size,
+                 interleaved=False, write_cache=True):
+        """Queries [rows, heads*head_dim], rotated, of f(x) . w^T; rotated keys and values go into the cache plane.
+
+        w: [(heads + 2 kv heads) * head_dim, K] with the rows of every q and k head in pair order. For few rows in
+        bfloat16 this is one kernel; otherwise the projection followed by the rotary/cache-write kernel.
+        """
+        _rows_view(self._check(x, "qkv x"), "qkv x")
+        self._check(w, "qkv w")
+        M, K = x.shape
+        N = (n_heads + 2 * n_kv_heads) * head_dim
+        if w.dim() != 2 or tuple(w.shape) != (N, K) or not w.is_contiguous():
+            raise KernelError(f"qkv_rope: w {tuple(w.shape)} is not [{N}, {K}] contiguous")
+        if self._skinny_ok(x, M, K) and head_dim % 4 == 0:
+            self._index(positions, "positions", M)
+            if table is not None:
+                self._check(table, "rotary table", torch.float32)
+                if table.dim() != 3 or table.shape[1] != head_dim // 2 or table.shape[2] != 2 or not table.is_contiguous():
+                    raise KernelError(f"qkv_rope: table {tuple(table.shape)} for head size {head_dim}")
+            if write_cache:
+                self._index(write_slots, "write_slots", M)
+                self._check_plane(plane, n_kv_heads, head_dim, page_size)
+            if rms is not None and (rms[0].numel() != K or rms[0].dtype != torch.float32):
+                raise KernelError(f"qkv_rope: norm gain has {rms[0].numel()} entries for width {K}")
+            q = self.empty(M, n_heads * head_dim)
+            self.gemm_skinny.tis_gemm_skinny_qkv_rope(
+                _ptr(x), x.stride(0), _ptr(w), _ptr(rms[0] if rms else None), float(rms[1]) if rms else 0.0, _ptr(q),
+                q.stride(0), M, K, _ptr(positions), _ptr(write_slots if write_cache else None), _ptr(table),
+                _ptr(plane if write_cache else None), n_heads, n_kv_heads, head_dim, page_size,
+                int(bool(interleaved)), int(bool(write_cache)), self._stream())
+            return q
+        qkv = self.linear(x, w, rms=rms)
+        q = self.empty(M, n_heads * head_dim)
+        self.rope_write_kv(qkv, positions, write_slots, table, plane, n_heads, n_kv_heads, head_dim, page_size,
+                           interleaved, write_cache, paired=True, q_out=q)
+        return q
 
     def _check_plane(self, plane, n_kv_heads, head_dim, page_size):
         self._check(plane, "cache plane")

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import MIXERS, build_part, normed_linear, to_compute
+from .base import MIXERS, build_part, to_compute
 from .spec import PagedKvNeed
 
 
@@ -41,8 +41,19 @@ class GqaAttention:
         self.scale = float(p.get("scale", self.head_dim ** -0.5))
         pos = p["position"]
         self.position = build_part(pos, tensors, ops)
-        # one projection for q, k and v: rows of the [out, in] matrix are q heads, then k heads, then v heads
-        self.w_qkv = to_compute(ops, torch.cat((tensors.of(spec, "q"), tensors.of(spec, "kv")), dim=1).t())
+        # one projection for q, k and v: rows of the [out, in] matrix are q heads, then k heads, then v heads.
+        # Inside every q and k head the rows are put in pair order (the two members of a rotary pair side by side),
+        # so that the kernel that makes them can rotate them while they are still in its registers.
+        w = torch.cat((tensors.of(spec, "q"), tensors.of(spec, "kv")), dim=1).t()
+        _, interleaved = self.position.rotary()
+        hd, half = self.head_dim, self.head_dim // 2
+        if not interleaved:
+            order = torch.stack((torch.arange(half), torch.arange(half) + half), dim=1).reshape(-1)
+            rows = torch.arange(w.shape[0]).view(-1, hd)
+            n_qk = self.n_heads + self.n_kv_heads
+            rows[:n_qk] = rows[:n_qk][:, order]
+            w = w[rows.reshape(-1)]
+        self.w_qkv = to_compute(ops, w)
         self.w_o = to_compute(ops, tensors.of(spec, "o").t())
         self.q_width = self.n_heads * self.head_dim
         if hasattr(ops, "register_attention"):
@@ -52,11 +63,16 @@ class GqaAttention:
 
     def forward(self, x, ctx, residual=None, norm=None):
         ops, b = self.ops, ctx.batch
-        qkv = normed_linear(ops, x, self.w_qkv, norm)
+        rms = None
+        if norm is not None:
+            if hasattr(norm, "as_rms"):
+                rms = norm.as_rms()
+            else:
+                x = norm(x)
         table, interleaved = self.position.rotary()
         page_size = ctx.plane.shape[3]
-        ops.rope_write_kv(qkv, b.positions, b.write_slots[ctx.group], table, ctx.plane, self.n_heads,
-                          self.n_kv_heads, self.head_dim, page_size, interleaved, ctx.writes_cache)
-        attn = ops.paged_attention(qkv[:, :self.q_width], ctx.plane, b, ctx.group, self.n_heads, self.n_kv_heads,
+        q = ops.qkv_rope(x, self.w_qkv, rms, b.positions, b.write_slots[ctx.group], table, ctx.plane, self.n_heads,
+                         self.n_kv_heads, self.head_dim, page_size, interleaved, ctx.writes_cache)
+        attn = ops.paged_attention(q, ctx.plane, b, ctx.group, self.n_heads, self.n_kv_heads,
                                    self.head_dim, self.window, self.scale)
         return ops.linear(attn, self.w_o, residual=residual)

@@ -40,7 +40,7 @@ __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cas
 __device__ __forceinline__ bf16x4 load4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
 
 template <int NB>
-__global__ __launch_bounds__(64) void attention_mfma_kernel(
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 : 1))) void attention_mfma_kernel(
     const bf16* __restrict__ q, long q_ld, const bf16* __restrict__ plane, const int* __restrict__ block_tables,
     int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ items,
     bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
@@ -82,6 +82,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
   int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
   k_lo &= ~31;
   const int k_hi = p_last + 1;
+  const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;   // the largest window start
   const int n_steps = (k_hi - k_lo + 31) / 32;
   const int per_split = (n_steps + n_splits - 1) / n_splits;
   const int s_begin = split * per_split;
@@ -159,9 +160,12 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
         for (int nb = 0; nb < NB; ++nb)
           st[t][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(T.k[t][dc], qb[nb][dc], st[t][nb], 0, 0, 0);
     }
-    // mask, running maximum and sum per column, P in bfloat16 as the B operand of the second product
+    // mask, running maximum and sum per column, P in bfloat16 as the B operand of the second product.
+    // A step whose 32 keys lie inside every column's range needs no mask at all (most steps of a long row).
+    const bool full = T.ok[0] && T.ok[1] && kb + 31 <= p_first && kb >= lo_last;
     bf16x8 pb[NB];
     float alpha[NB];
+    bool grew = false;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       float sv[8];
@@ -170,22 +174,31 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int key = kb + t * 16 + g * 4 + i;
-          const bool ok = T.ok[t] && key <= col_pos[nb] && key >= col_lo[nb];
-          const float v = ok ? st[t][nb][i] * scale_log2 : -INFINITY;
+          float v = st[t][nb][i] * scale_log2;
+          if (!full) {
+            const int key = kb + t * 16 + g * 4 + i;
+            const bool ok = T.ok[t] && key <= col_pos[nb] && key >= col_lo[nb];
+            v = ok ? v : -INFINITY;
+          }
           sv[t * 4 + i] = v;
           tmax = fmaxf(tmax, v);
         }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m[nb], tmax);
+      // m is the exponent that P, the sum and the output are taken relative to. It follows the running maximum
+      // only when that has grown by more than 2^8 beyond it, so it settles after a row's first keys and the
+      // rescaling below becomes rare; until then P stays below 256, well inside bfloat16, and sum and output
+      // share the factor, which cancels in their ratio.
+      const bool move = tmax > m[nb] + 8.f || m[nb] == -INFINITY;
+      const float m_new = move ? fmaxf(m[nb], tmax) : m[nb];
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a column with no key yet: everything stays 0
-      alpha[nb] = exp2f(m[nb] - m_use);
+      grew = grew || (move && m_new > m[nb]);
+      alpha[nb] = __builtin_amdgcn_exp2f(m[nb] - m_use);
       float psum = 0.f;
       bf16x8 pv;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = exp2f(sv[e] - m_use);
+        const float p = __builtin_amdgcn_exp2f(sv[e] - m_use);   // arguments are <= 8: no overflow to guard
         psum += p;
         pv[e] = static_cast<__bf16>(p);
       }
@@ -193,19 +206,39 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
       l[nb] = l[nb] * alpha[nb] + psum;      // the lane's share; the four key groups are added at the end
       m[nb] = m_new;
     }
-    // O^T = O^T * alpha + V^T . P^T
+    // O^T = O^T * alpha + V^T . P^T. The running maximum settles after the first keys of a row; while no
+    // column of the wave has a new maximum every alpha is exactly 1 and the accumulators are left alone.
+    if (__builtin_amdgcn_ballot_w64(grew) != 0) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[nb][db][i] *= alpha[nb];
+    }
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        f32x4 acc = o[nb][db];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] *= alpha[nb];
-        o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(T.v[db], pb[nb], acc, 0, 0, 0);
-      }
+      for (int nb = 0; nb < NB; ++nb)
+        o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(T.v[db], pb[nb], o[nb][db], 0, 0, 0);
   };
 
-  if (s_begin < s_end) {
+  if (NB >= 2) {
+    // Wide items (rows of prompt portions) are bound by arithmetic, not by memory: they keep one step's tiles only,
+    // which leaves registers for a second wave per SIMD to fill the gaps, and prefetch just the page ids.
+    if (s_begin < s_end) {
+      Tiles ta;
+      int pa[2], pn[2];
+      page_ids(s_begin, pa);
+      for (int s = s_begin; s < s_end; ++s) {
+        load_tiles(s, pa, ta);
+        page_ids(s + 1, pn);
+        consume(s, ta);
+        pa[0] = pn[0];
+        pa[1] = pn[1];
+      }
+    }
+  } else if (s_begin < s_end) {
     Tiles ta, tb;
     int pa[2], pn[2], pq[2];
     page_ids(s_begin, pa);
@@ -339,7 +372,7 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
   if (n_splits > 1) {
     dim3 mgrid(rows, n_heads);
     attention_merge_kernel<<<mgrid, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld, n_heads,
-                                                     n_splits);
+                                                          n_splits);
     rc = tis_launch_status("attention_merge");
   }
   return rc;

@@ -120,3 +120,21 @@ def test_all_schedules_agree_with_each_other(backend):
         assert other.keys() == outs[0].keys()
         worst = max((other[k] - outs[0][k]).abs().max().item() for k in other)
         assert worst <= 2e-5
+
+
+@pytest.mark.gpu
+def test_long_context_decoding_in_bfloat16():
+    """A prompt of 500 tokens in uneven portions, then 120 tokens one by one through captured graphs: keys are cut
+    into several splits, pages are crossed, and every logit still matches the plain model."""
+    name, dtype = "D", "bfloat16"
+    reqs = requests_for(name, [620], seed=8)
+    folder, eng = make_engine(name, dtype, "hip", max_tokens=640)
+    ids = reqs["r0"]
+    steps, p = [], 0
+    for n in [333, 100, 67] + [1] * 120:
+        steps.append({"step": len(steps), "entries": [{"id": "r0", "tokens": ids[p:p + n], "want": [n - 1] if n > 1 else [0]}],
+                      "end": []})
+        p += n
+    main, _ = H.run_trace(eng, steps, heads=False)
+    assert eng.graph_replays >= 100
+    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0)

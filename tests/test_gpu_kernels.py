@@ -294,7 +294,26 @@ def test_sampling_reference_vectors(ops_for):
     assert ops.sample(lg.cuda(), *args, one(2.0), one(0.5), one(5, torch.int32), torch.tensor([0, 1], dtype=torch.int32).cuda()).item() == 7
 
 
-@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("M", [17, 64, 200])
+@pytest.mark.parametrize("N,K", [(96, 64), (1000, 96), (2304, 1536)])
+def test_product_with_norm_residual_and_gate_for_many_rows(ops_for, M, N, K):
+    """Above 16 rows the same calls run as separate kernels around the library's product; the results agree with the
+    reference's order of operations (norm rounded to bfloat16, product, gating)."""
+    ops, ref = ops_for(torch.bfloat16), TorchOps(dtype=torch.bfloat16)
+    x, w, res = rnd((M, K), torch.bfloat16, 80, 2.0), rnd((N, K), torch.bfloat16, 81, K ** -0.5), rnd((M, N), torch.bfloat16, 82)
+    gain = 1 + 0.1 * rnd((K,), torch.float32, 83)
+    t = dict(rtol=2e-2, atol=2e-2)
+    xn = ref.rmsnorm(x, gain, 1e-5).double()
+    torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), xn @ w.double().t(), **t)
+    torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), residual=res.cuda()).cpu().double(),
+                               x.double() @ w.double().t() + res.double(), **t)
+    gu = (xn @ w.double().t()).to(torch.bfloat16).double()
+    want = torch.nn.functional.silu(gu[:, 0::2]) * gu[:, 1::2]
+    torch.testing.assert_close(ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), want,
+                               rtol=3e-2, atol=3e-2)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16])
 @pytest.mark.parametrize("N,K", [(96, 64), (1000, 96), (130, 264), (2304, 1536), (1536, 4096)])
 def test_skinny_product_with_fused_norm_residual_and_gate(ops_for, M, N, K):
     """The few-row matrix-core product and what is fused around it, against the unfused plain computation."""
@@ -325,7 +344,7 @@ def test_skinny_product_with_fused_norm_residual_and_gate(ops_for, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M", [1, 5, 64, 200])
+@pytest.mark.parametrize("M", [1, 5, 16, 64, 200])
 @pytest.mark.parametrize("n_heads,n_kv,hd,page_size,interleaved", [(8, 2, 8, 16, False), (3, 1, 32, 8, False),
                                                                     (12, 3, 128, 16, False), (4, 2, 48, 16, True)])
 def test_projection_with_rotary_and_cache_write(ops_for, dtype, M, n_heads, n_kv, hd, page_size, interleaved):

@@ -204,3 +204,60 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
             assert (lg.double() - want).abs().max() <= 2e-5 * max(1.0, want.abs().max()), (rid, p)
     ARCHITECTURES.unregister("ToyStateModel")
     MIXERS.unregister("toy_decay")
+
+
+# ---- layers with different cache needs in one model: a sliding window beside full attention ----------------------
+
+def windowed_spec(cfg, windows):
+    from tiny_inference_server_amd.architectures.gqa_mtp import _block, _norm
+    import dataclasses
+    layers = []
+    for l, win in enumerate(windows):
+        blk = _block(cfg, f"transformer_block_list.{l}.")
+        mixer = dataclasses.replace(blk.mixer, params={**blk.mixer.params, "window": win})
+        layers.append(dataclasses.replace(blk, mixer=mixer))
+    stage = StageSpec("trunk", 0, PartSpec("stage_input", "token_embedding"), tuple(LayerCall(l) for l in range(len(windows))),
+                      _norm(cfg, "rms_out.scale"))
+    return ModelSpec(cfg.d_model, cfg.vocab_size, cfg.max_context, tuple(layers), (stage,), "embedding.weight", "embedding.weight")
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 2e-2)])
+def test_window_layers_get_pages_of_their_own_and_give_them_back(dtype, tol):
+    """Layer 0 sees the last 24 keys, layer 1 all of them, layer 2 the last 40: three page groups. Window groups hold
+    few pages however long the request grows, and the logits equal the plain model's with the same windows."""
+    from tiny_inference_server_amd.config import GqaMtpConfig
+    windows = (24, 0, 40)
+    cfg = GqaMtpConfig(d_model=128, vocab_size=211, max_context=512, rope_base=1e4, n_heads=4, n_layers=3, ffn_hidden=160,
+                       group_size=2, mtp_heads=0, architecture="WindowedToy")
+    ARCHITECTURES.register("WindowedToy", Architecture("WindowedToy", GqaMtpConfig, lambda c: windowed_spec(c, windows)),
+                           replace=True)
+    w = random_tensors(cfg, 21, std=0.08, gain_jitter=0.1, dtype=dtype)
+    eng = Engine(config=cfg, tensors=w, dtype=dtype, page_size=16, max_tokens=512, max_requests=2)
+    assert len(eng.cache.groups) == 3
+    ids = H.random_ids(211, 300, 5)
+    # plain: the same blocks with their windows
+    w64 = {k: v.double() for k, v in w.items()}
+    pcfg = {"n_heads": 4, "group": 2, "eps": cfg.rms_eps, "base": 1e4}
+    x = w64["embedding.weight"][torch.tensor(ids)]
+    for l, win in enumerate(windows):
+        x = pm.block(x, w64, f"transformer_block_list.{l}.", pcfg, torch.arange(len(ids)), window=win)
+    want = pm.rms_norm(x, w64["rms_out.scale"], cfg.rms_eps) @ w64["embedding.weight"].T
+    # a long portion, portions that end inside and on page edges, then token by token
+    got, p = {}, 0
+    for n in [100, 37, 27, 16, 1, 1, 30] + [1] * 88:
+        out = eng.step([("a", ids[p:p + n], list(range(n)))])
+        lg = out.logits.float().cpu()
+        for i in range(n):
+            got[p + i] = lg[i]
+        p += n
+        held = {name: g.held(eng.requests["a"][0]) for name, g in eng.cache.groups.items()}
+        assert held["kv2x32"] == -(-p // 16)
+        assert held["kv2x32w24"] <= 24 // 16 + 2 and held["kv2x32w40"] <= 40 // 16 + 2
+    assert p == 300
+    scale = max(1.0, want.abs().max().item())
+    worst = max((got[i].double() - want[i]).abs().max().item() for i in range(300))
+    assert worst <= tol * scale, worst
+    eng.close("a")
+    eng.cache.check()
+    assert all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups.values())
+    ARCHITECTURES.unregister("WindowedToy")

@@ -1,4 +1,4 @@
-// C[M,N] = f(A[M,K]) . W[N,K]^T for few rows (M <= 64): the matrix product of decode steps, where the job is to
+// C[M,N] = f(A[M,K]) . W[N,K]^T for few rows (M <= 16): the matrix product of decode steps, where the job is to
 // stream W from HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950).
 //
 // One workgroup owns 16 rows of W (16 output columns) over the whole of K; its waves take the 32-wide steps of
@@ -222,9 +222,9 @@ static void launch(const void* X, long x_ld, const void* W, const float* gain, f
 template <bool NORM, int EPI, typename TO>
 static int launch_mb(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
                      void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope = RopeArgs()) {
-  if (M <= 16) launch<1, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
-  else if (M <= 32) launch<2, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
-  else launch<4, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
+  // one block of 16 rows: with more rows the library's product is faster than this kernel even after paying for
+  // the separate norm, gating and rotary launches, so more blocks (MB > 1) are not built
+  launch<1, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
   return tis_launch_status("gemm_skinny");
 }
 
@@ -233,7 +233,7 @@ TIS_EXPORT int tis_gemm_skinny(const void* X, long x_ld, const void* W, const fl
                                long r_ld, void* C, long c_ld, int M, int N, int K, int epilogue, int out_dtype,
                                hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
-  if (M < 0 || M > 64) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..64", M);
+  if (M < 0 || M > 16) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..16", M);
   if (N < 1 || K < 8 || K % 8) return tis_fail("gemm_skinny: N=%d K=%d; K must be a multiple of 8", N, K);
   if (x_ld % 8 || ((uintptr_t)X % 16) || ((uintptr_t)W % 16))
     return tis_fail("gemm_skinny: activations and weights must be 16-byte aligned with row strides in steps of 8");
@@ -259,7 +259,7 @@ TIS_EXPORT int tis_gemm_skinny_qkv_rope(const void* X, long x_ld, const void* W,
                                         const float* table, void* plane, int n_heads, int n_kv_heads, int head_dim,
                                         int page_size, int interleaved, int write_cache, hipStream_t stream) {
   if (M == 0) return 0;
-  if (M < 0 || M > 64) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..64", M);
+  if (M < 0 || M > 16) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..16", M);
   if (K < 8 || K % 8) return tis_fail("gemm_skinny: K=%d must be a multiple of 8", K);
   if (n_heads < 1 || n_kv_heads < 1 || head_dim < 4 || head_dim % 4 || page_size < 1)
     return tis_fail("gemm_skinny: heads=%d kv_heads=%d head_dim=%d (a multiple of 4) page=%d", n_heads, n_kv_heads,

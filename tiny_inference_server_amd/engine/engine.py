@@ -178,9 +178,15 @@ class Engine:
         pages = max((max(len(g.tables[e.slot]) for e in batch_entries) for g in self.cache.groups.values()), default=1)
         width = -(-pages // self.graph_table_pages) * self.graph_table_pages
         key = (len(batch_entries), width)
+        graph = self._graphs.get(key)
+        if graph is not None and graph.slots == tuple(e.slot for e in batch_entries):
+            for e in batch_entries:
+                if e.start + 1 > self.spec.max_context:
+                    raise ValueError(f"request in slot {e.slot} would pass the model's context of {self.spec.max_context}")
+            self.graph_replays += 1
+            return graph.run_same_requests(batch_entries)
         plan = plan_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
                                self.spec.max_context, getattr(self.ops, "plan_rows", None), table_width=width)
-        graph = self._graphs.get(key)
         if graph is None:
             seen = self._graph_seen.get(key, 0)
             self._graph_seen[key] = seen + 1

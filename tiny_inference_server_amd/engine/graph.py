@@ -11,6 +11,7 @@ also sizes the kernels' workspace), so a capture records kernel launches only.
 """
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from .batch import StepPlan, materialize
@@ -33,6 +34,48 @@ class DecodeGraph:
             outs = engine.model.forward(self.step, engine.cache)
             self.logits = engine.model.logits(outs[0].hidden, self.step.stages[0].want_index, n)
         self.copied.record()
+        # what the quick update needs: which requests, in which order, the buffer holds, and where their arrays lie
+        self.slots = tuple(e.slot for e in plan.entries)
+        self.cache = engine.cache
+        self.page_size = engine.page_size
+        off = lambda i: plan.packer.offsets[i][0]
+        self.table_at = {g: (off(i), plan.packer.offsets[i][1]) for g, i in plan.bt_ids.items()}
+        self.stage_at = [dict(lag=pl["lag"], tokens=off(pl["tokens"]), positions=off(pl["positions"]),
+                              ws={g: off(i) for g, i in pl["ws"].items()}) for pl in plan.plans]
+        self.pages_held = {g: np.array([len(engine.cache.groups[g].tables[s]) for s in self.slots])
+                           for g in self.table_at}
+
+    def run_same_requests(self, entries) -> torch.Tensor:
+        """The next step of the very requests whose arrays the buffer already holds, in the same order: only
+        tokens, positions, write slots and newly taken pages change, and those are written in place."""
+        self.copied.synchronize()
+        flat = self.host.numpy()
+        n = len(entries)
+        starts = np.fromiter((e.start for e in entries), dtype=np.int64, count=n)
+        tokens = np.fromiter((e.tokens[0] for e in entries), dtype=np.int32, count=n)
+        ps = self.page_size
+        for g, (t_off, (rows, width)) in self.table_at.items():
+            tables = self.cache.groups[g].tables
+            need = starts // ps + 1
+            for k in np.nonzero(need > self.pages_held[g])[0]:
+                t = tables[self.slots[k]]
+                if len(t) > width:
+                    raise RuntimeError("a block table outgrew the captured width")
+                flat[t_off + k * width:t_off + k * width + len(t)] = [p if p >= 0 else 0 for p in t]
+                self.pages_held[g][k] = len(t)
+        rows_idx = np.arange(n)
+        for st in self.stage_at:
+            pos = starts - st["lag"]
+            flat[st["tokens"]:st["tokens"] + n] = tokens
+            flat[st["positions"]:st["positions"] + n] = pos
+            for g, w_off in st["ws"].items():
+                t_off, (rows, width) = self.table_at[g]
+                table = flat[t_off:t_off + rows * width].reshape(rows, width)
+                flat[w_off:w_off + n] = table[rows_idx, pos // ps] * ps + pos % ps
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+        self.graph.replay()
+        return self.logits
 
     def run(self, plan: StepPlan) -> torch.Tensor:
         if plan.layout() != self.layout:
@@ -41,5 +84,8 @@ class DecodeGraph:
         plan.packer.fill(self.host)
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
+        self.slots = tuple(e.slot for e in plan.entries)
+        for g in self.table_at:
+            self.pages_held[g] = np.array([len(self.cache.groups[g].tables[s]) for s in self.slots])
         self.graph.replay()
         return self.logits

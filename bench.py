@@ -23,7 +23,7 @@ sys.path.insert(0, ROOT)
 HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 # the reference's plain decode at batch 8 on an A6000: 31.7 ms per iteration of 8 tokens (README.md:325)
-BASELINE_B8_TOKS = 8 / 31.7e-3
+REFERENCE_B8_TOKS = 8 / 31.7e-3
 
 
 def matmul_params(cfg, heads: bool):
@@ -152,7 +152,7 @@ def main() -> int:
         "metric": "decode tok/s at batch 8 (0.9B, bf16); prefill tok/s at 2,048 tokens",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(sec_per_step * 1e3, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": round(value / BASELINE_B8_TOKS, 2) if (a.batch == 8 and a.size == "0.9B") else None,
+        "vs_baseline": round(value / REFERENCE_B8_TOKS, 2) if (a.batch == 8 and a.size == "0.9B") else None,
         "dtype": dkey, "data": "synthetic: random weights N(0,0.02), uniform random token ids",
         "config": {
             "model": a.size, "global_batch": a.batch, "seq_len": a.context, "parallelism": "single-gpu",

@@ -19,7 +19,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_greedy_generation_equals_plain(name):
-    """BASELINE's tiny workloads: 3 prompts of 5/17/33 tokens, 16 greedy tokens each (A); 1/9/24/40 (B)."""
+    """Two tiny workloads: 3 prompts of 5/17/33 tokens (A) and 4 of 1/9/24/40 tokens (B), 16 greedy tokens each."""
     folder = H.model_folder(name, "float32")
     cfg, w = pm.read_model_folder(folder)
     lens = [5, 17, 33] if name == "A" else [1, 9, 24, 40]

@@ -60,7 +60,7 @@ class TorchOps:
             return out
         return y
 
-    def linear(self, x, w, residual=None, out_dtype=None, rms=None):
+    def linear(self, x, w, residual=None, out_dtype=None, rms=None, reuse_residual=False):
         if rms is not None:
             x = self.rmsnorm(x, rms[0], rms[1])
         y = x.float() @ w.float().t()

@@ -79,7 +79,8 @@ class Model:
                 for i, call in enumerate(st.calls):
                     key = self.call_keys[j][i]
                     need = self.needs.get(key)
-                    ctx = CallContext(batch=b, writes_cache=call.writes_cache)
+                    # the rows going into a layer are replaced by its result: the layer may overwrite them
+                    ctx = CallContext(batch=b, writes_cache=call.writes_cache, residual_is_spent=True)
                     if isinstance(need, PagedKvNeed):
                         ctx.group = cache.group_of[key]
                         ctx.plane = cache.groups[ctx.group].plane(key)

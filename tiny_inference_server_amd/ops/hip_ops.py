@@ -285,10 +285,12 @@ class HipOps:
         return out
 
     # ---- matrix products -----------------------------------------------------------------------------
-    def linear(self, x, w, residual=None, out_dtype=None, rms=None):
+    def linear(self, x, w, residual=None, out_dtype=None, rms=None, reuse_residual=False):
         """f(x)[M,K] . w[N,K]^T (+ residual[M,N]); `out_dtype` float32 gives 32-bit results from bfloat16 inputs.
 
         rms = (gain, eps): f is the RMSNorm of the rows, fused into the product where the kernel allows.
+        reuse_residual: the caller has no further use for `residual`, so the result may be written over it
+        (the library's product then adds in place instead of copying the residual first).
         """
         _rows_view(self._check(x, "linear x"), "linear x")
         self._check(w, "linear w")
@@ -320,7 +322,7 @@ class HipOps:
                                            residual.stride(0) if residual is not None else 0, _ptr(out), N, M, N, K,
                                            self._stream())
             return out
-        return self._linear_bf16(x, w, residual, out_dtype)
+        return self._linear_bf16(x, w, residual, out_dtype, reuse_residual)
 
     def _skinny_ok(self, x, M, K):
         # up to 16 rows the fused few-row kernel wins (it saves the norm, gating and rotary launches and streams the
@@ -346,13 +348,15 @@ class HipOps:
             return out
         return self.swiglu(self.linear(x, w, rms=rms))
 
-    def _linear_bf16(self, x, w, residual, out_dtype):
+    def _linear_bf16(self, x, w, residual, out_dtype, reuse_residual=False):
         if out_dtype == torch.float32:
             out = torch.matmul(x, w.t()).float()
             if residual is not None:
                 out += residual
             return out
         if residual is not None:
+            if reuse_residual and residual.is_contiguous():
+                return torch.addmm(residual, x, w.t(), out=residual)
             return torch.addmm(residual, x, w.t())
         return torch.matmul(x, w.t())
 

@@ -75,4 +75,4 @@ class GqaAttention:
                          self.n_kv_heads, self.head_dim, page_size, interleaved, ctx.writes_cache)
         attn = ops.paged_attention(q, ctx.plane, b, ctx.group, self.n_heads, self.n_kv_heads,
                                    self.head_dim, self.window, self.scale)
-        return ops.linear(attn, self.w_o, residual=residual)
+        return ops.linear(attn, self.w_o, residual=residual, reuse_residual=ctx.residual_is_spent)

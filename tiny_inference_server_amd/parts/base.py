@@ -50,6 +50,7 @@ class CallContext:
     plane: Any = None                # [pages, 2, kv heads, page size, head size] for paged needs
     state: Any = None                # [max requests, *shape] for state needs
     writes_cache: bool = True
+    residual_is_spent: bool = False  # the caller will not read the residual it passes again: it may be overwritten
 
 
 class Tensors:

@@ -15,10 +15,12 @@ class PreNormResidual:
         self.ffn = build_part(layer_spec.feed_forward, tensors, ops)
 
     def forward(self, x, ctx):
+        # the stream `x` is replaced by each sub-layer's result, so the residual passed down is spent and a part may
+        # write its result over it; whether the block's own input is spent too, the caller says in ctx
         if getattr(self.mixer, "fuses_norm", False):
             x = self.mixer.forward(x, ctx, residual=x, norm=self.mixer_norm)
         else:
             x = self.mixer.forward(self.mixer_norm(x), ctx, residual=x)
         if getattr(self.ffn, "fuses_norm", False):
-            return self.ffn.forward(x, residual=x, norm=self.ffn_norm)
+            return self.ffn.forward(x, residual=x, norm=self.ffn_norm, residual_is_spent=True)
         return self.ffn.forward(self.ffn_norm(x), residual=x)

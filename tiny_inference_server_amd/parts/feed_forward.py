@@ -30,9 +30,9 @@ class SwiGlu:
 
     fuses_norm = True
 
-    def forward(self, x, residual=None, norm=None):
+    def forward(self, x, residual=None, norm=None, residual_is_spent=False):
         ops = self.ops
         if norm is not None and not hasattr(norm, "as_rms"):
             x, norm = norm(x), None
         hidden = ops.linear_swiglu(x, self.w_gate_up, rms=norm.as_rms() if norm is not None else None)
-        return ops.linear(hidden, self.w_down, residual=residual)
+        return ops.linear(hidden, self.w_down, residual=residual, reuse_residual=residual_is_spent)

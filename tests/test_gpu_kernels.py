@@ -377,3 +377,35 @@ def test_projection_with_rotary_and_cache_write(ops_for, dtype, M, n_heads, n_kv
         c, s = table[positions.long()][..., 0].double().repeat(1, 2).unsqueeze(1), table[positions.long()][..., 1].double().repeat(1, 2).unsqueeze(1)
         rot = torch.cat((-q[..., half:], q[..., :half]), dim=-1)
         torch.testing.assert_close(got.double().view(M, n_heads, hd), q * c + rot * s, **t)
+
+
+def test_sampling_with_the_context_kept_on_the_device(ops_for):
+    """The penalty's context as a byte table per request instead of a token list: same draws, and the kernel marks
+    what it drew."""
+    ops = ops_for(torch.float32)
+    n, V = 5, 777
+    logits = rnd((n, V), torch.float32, 90, 3.0)
+    temperature = torch.tensor([0.0, 1.0, 0.8, 1.0, 0.9])
+    top_k = torch.tensor([0, 40, 0, 3, 50], dtype=torch.int32)
+    top_p = torch.tensor([0.0, 0.9, 0.0, 0.9, 0.95])
+    pen = torch.tensor([1.5, 1.2, 1.0, 1.3, 1.1])
+    ctx = [torch.tensor(sorted(set(random.Random(91 + i).choices(range(V), k=30))), dtype=torch.int32) for i in range(n)]
+    off = torch.tensor([0] + list(torch.tensor([len(c) for c in ctx]).cumsum(0)), dtype=torch.int32)
+    u = torch.rand(n, generator=torch.Generator().manual_seed(92))
+    by_list = ops.sample(logits.cuda(), temperature.cuda(), top_k.cuda(), top_p.cuda(), pen.cuda(), u.cuda(),
+                         torch.cat(ctx).cuda(), off.cuda()).cpu()
+    seen = torch.zeros(8, V, dtype=torch.uint8)
+    lines = torch.tensor([6, 0, -1, 3, 2], dtype=torch.int32)          # row 2 has no penalty and no line
+    for i in range(n):
+        if lines[i] >= 0:
+            seen[lines[i], ctx[i].long()] = 1
+    seen_gpu = seen.cuda()
+    by_table = ops.sample(logits.cuda(), temperature.cuda(), top_k.cuda(), top_p.cuda(), pen.cuda(), u.cuda(),
+                          seen=seen_gpu, seen_row=lines.cuda()).cpu()
+    assert by_table.tolist() == by_list.tolist()
+    after = seen_gpu.cpu()
+    for i in range(n):
+        if lines[i] >= 0:
+            want = seen[lines[i]].clone(); want[by_table[i]] = 1
+            assert torch.equal(after[lines[i]], want)
+    assert torch.equal(after[[1, 4, 5, 7]], seen[[1, 4, 5, 7]])

@@ -144,10 +144,22 @@ class TorchOps:
     def argmax(self, logits):
         return torch.argmax(logits, dim=-1).to(torch.int32)
 
-    def sample(self, logits, temperature, top_k, top_p, rep_penalty, uniform, ctx_tokens=None, ctx_offsets=None):
+    def sample(self, logits, temperature, top_k, top_p, rep_penalty, uniform, ctx_tokens=None, ctx_offsets=None,
+               seen=None, seen_row=None):
         """The kernel's method: thresholds instead of a sort, inverse CDF in token order."""
         n, V = logits.shape
         out = torch.zeros(n, dtype=torch.int32)
+        if seen is not None:
+            # the byte-table form of the context: turn each row's line into a token list, mark the draw afterwards
+            lists = [torch.nonzero(seen[int(seen_row[r])]).flatten().to(torch.int32) if int(seen_row[r]) >= 0
+                     else torch.zeros(0, dtype=torch.int32) for r in range(n)]
+            offs = torch.tensor([0] + list(torch.tensor([len(l) for l in lists]).cumsum(0)), dtype=torch.int32)
+            flat = torch.cat(lists) if lists else torch.zeros(0, dtype=torch.int32)
+            out = self.sample(logits, temperature, top_k, top_p, rep_penalty, uniform, flat, offs)
+            for r in range(n):
+                if int(seen_row[r]) >= 0:
+                    seen[int(seen_row[r]), int(out[r])] = 1
+            return out
         for r in range(n):
             l = logits[r].float().clone()
             t, k, p = float(temperature[r]), int(top_k[r]), float(top_p[r])

@@ -4,9 +4,9 @@
 // tokens of the request's context (l > 0 ? l / pen : l * pen, each token once) -> divide by the
 // temperature -> top-k -> top-p (keep a token while the probability mass of the strictly larger ones is
 // <= top_p, so the token that crosses top_p stays) -> softmax over what is left -> draw.
-// The reference sorts; here both cuts are thresholds found by bisection over the bit pattern of the
-// values, which keeps the same set whenever the values at the cut are distinct (ties at the top-k cut
-// are all kept). The draw takes a uniform number per row from the caller (a stream per request, so a
+// The reference sorts; here both cuts are thresholds over the bit pattern of the values (a radix select for
+// top-k, then the few survivors are handled in LDS; a bisection for top-p without top-k), which keeps the
+// same set whenever the values at the cut are distinct (ties at the top-k cut are all kept). The draw takes a uniform number per row from the caller (a stream per request, so a
 // request's tokens do not depend on what else is in the batch) and inverts the cumulative distribution
 // in token order. temperature == 0 or top_k == 1 is greedy: the arg-max, lowest index on ties.
 #include "common.h"
@@ -41,13 +41,19 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
     const float* __restrict__ logits, long ld, float* __restrict__ work, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ rep_penalty,
     const int* __restrict__ ctx_tokens, const int* __restrict__ ctx_offsets, const float* __restrict__ uniform,
-    int* __restrict__ out_tokens) {
+    int* __restrict__ out_tokens, unsigned char* __restrict__ seen, long seen_ld, const int* __restrict__ seen_row) {
   __shared__ float red[16];
   __shared__ float sv[16];
   __shared__ int si[16];
   __shared__ float part[SM_THREADS];
   __shared__ int found;
   __shared__ int first_owner;
+  __shared__ unsigned hist[256];
+  __shared__ int sel_bin, sel_rem, n_cand;
+  __shared__ int icount[SM_THREADS];
+  __shared__ float cand_e[SM_THREADS];
+  __shared__ float cand_v[SM_THREADS];
+  __shared__ int cand_i[SM_THREADS];
 
   const long r = blockIdx.x;
   const int t = threadIdx.x;
@@ -62,7 +68,19 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
 
   for (int i = t; i < V; i += SM_THREADS) x[i] = lg[i] * inv_t;
   __syncthreads();
-  if (pen != 1.f && ctx_tokens) {
+  // The request's context comes either as a list of tokens or as a row of a table with one byte per token of
+  // the vocabulary (nonzero: the token has occurred); the table's row also gets the token drawn here, so that a
+  // server only ever uploads a request's context once.
+  unsigned char* mark = (seen && seen_row && seen_row[r] >= 0) ? seen + (long)seen_row[r] * seen_ld : nullptr;
+  if (pen != 1.f && mark) {
+    for (int i = t; i < V; i += SM_THREADS) {
+      if (mark[i]) {
+        const float l = lg[i];
+        x[i] = (l > 0.f ? l / pen : l * pen) * inv_t;
+      }
+    }
+    __syncthreads();
+  } else if (pen != 1.f && ctx_tokens) {
     // computed from the untouched logits, so a token that occurs twice is still penalised once
     for (int c = ctx_offsets[r] + t; c < ctx_offsets[r + 1]; c += SM_THREADS) {
       const int tok = ctx_tokens[c];
@@ -84,21 +102,125 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
   block_argmax(mv, mi, sv, si);
   if (mi < 0 || mi >= V) mi = 0;  // only when every value is NaN
   if (greedy) {
-    if (t == 0) out_tokens[r] = mi;
+    if (t == 0) {
+      out_tokens[r] = mi;
+      if (mark) mark[mi] = 1;
+    }
     return;
   }
 
-  // top-k: the k-th largest key, built bit by bit
+  // top-k: the k-th largest key by a radix select, eight bits a pass over a histogram of counts in LDS
+  // (integer counts, so the result does not depend on the order in which threads arrive)
   unsigned cut = 0u;
-  if (k_req > 0 && k_req < V) {
-    for (int bit = 31; bit >= 0; --bit) {
-      const unsigned cand = cut | (1u << bit);
-      float cnt = 0.f;
-      for (int i = t; i < V; i += SM_THREADS) cnt += (order_key(x[i]) >= cand) ? 1.f : 0.f;
-      cnt = block_sum(cnt, red);
-      if (cnt >= (float)k_req) cut = cand;
+  const bool has_k = k_req > 0 && k_req < V;
+  if (has_k) {
+    unsigned prefix = 0u;
+    int remaining = k_req;
+    for (int pass = 0; pass < 4; ++pass) {
+      const int shift = 24 - 8 * pass;
+      if (t < 256) hist[t] = 0u;
+      __syncthreads();
+      for (int i = t; i < V; i += SM_THREADS) {
+        const unsigned key = order_key(x[i]);
+        if (pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8))) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      if (t == 0) {
+        int seen = 0, b = 255;
+        for (; b > 0; --b) {
+          if (seen + (int)hist[b] >= remaining) break;
+          seen += (int)hist[b];
+        }
+        sel_bin = b;
+        sel_rem = remaining - seen;
+      }
+      __syncthreads();
+      prefix |= (unsigned)sel_bin << shift;
+      remaining = sel_rem;
+      __syncthreads();
+    }
+    cut = prefix;
+  }
+
+  // With a top-k cut the survivors are few: gather them, in token order, into LDS and finish there.
+  const int chunk = (V + SM_THREADS - 1) / SM_THREADS;
+  const int lo = min(V, t * chunk), hi = min(V, lo + chunk);
+  if (has_k) {
+    int mine_n = 0;
+    for (int i = lo; i < hi; ++i) mine_n += order_key(x[i]) >= cut ? 1 : 0;
+    // exclusive scan of the 1024 counts, in thread order: sixteen per lane of the first wave, then across its lanes
+    icount[t] = mine_n;
+    __syncthreads();
+    if (t < TIS_WAVE) {
+      int s = 0;
+      for (int i = 0; i < SM_THREADS / TIS_WAVE; ++i) s += icount[t * (SM_THREADS / TIS_WAVE) + i];
+      int incl = s;
+#pragma unroll
+      for (int o = 1; o < TIS_WAVE; o <<= 1) {
+        const int up = __shfl_up(incl, o, TIS_WAVE);
+        if (t >= o) incl += up;
+      }
+      int run = incl - s;
+      for (int i = 0; i < SM_THREADS / TIS_WAVE; ++i) {
+        const int ix = t * (SM_THREADS / TIS_WAVE) + i;
+        const int v = icount[ix];
+        icount[ix] = run;
+        run += v;
+      }
+      if (t == TIS_WAVE - 1) n_cand = run;
+    }
+    __syncthreads();
+    const int n = n_cand;
+    if (n <= SM_THREADS) {     // more only when many values tie at the cut: then the general path below takes over
+      int at = icount[t];
+      for (int i = lo; i < hi; ++i) {
+        const float v = x[i];
+        if (order_key(v) >= cut) {
+          cand_e[at] = expf(v - mv);
+          cand_v[at] = v;
+          cand_i[at] = i;
+          ++at;
+        }
+      }
+      __syncthreads();
+      // top-p on the survivors: keep one while the mass of the strictly larger ones is <= top_p of the whole
+      float zk = 0.f;
+      for (int j = 0; j < n; ++j) zk += cand_e[j];
+      bool keep = t < n;
+      if (keep && p_req > 0.f && p_req < 1.f) {
+        float above = 0.f;
+        for (int j = 0; j < n; ++j) above += cand_v[j] > cand_v[t] ? cand_e[j] : 0.f;
+        keep = above <= p_req * zk;
+      }
+      __syncthreads();
+      if (t < n && !keep) cand_e[t] = 0.f;
+      __syncthreads();
+      // inverse CDF in token order; every thread adds the same numbers in the same order, so the intervals
+      // [before, before + e) of neighbours meet exactly
+      float zz = 0.f, before = 0.f;
+      for (int j = 0; j < n; ++j) {
+        if (j == t) before = zz;
+        zz += cand_e[j];
+      }
+      const float target = uniform[r] * zz;
+      if (t == 0) found = -1;
+      __syncthreads();
+      if (t < n && cand_e[t] > 0.f && before <= target && target < before + cand_e[t]) found = cand_i[t];
+      __syncthreads();
+      if (t == 0) {
+        int pick = found;
+        if (pick < 0) {          // rounding left the target at the very end: the last survivor
+          for (int j = n - 1; j >= 0 && pick < 0; --j)
+            if (cand_e[j] > 0.f) pick = cand_i[j];
+        }
+        pick = pick >= 0 ? pick : mi;
+        out_tokens[r] = pick;
+        if (mark) mark[pick] = 1;
+      }
+      return;
     }
   }
+
   float z = 0.f;
   for (int i = t; i < V; i += SM_THREADS) {
     const float v = x[i];
@@ -133,8 +255,6 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
   }
 
   // inverse CDF in token order: thread t owns the tokens [t*chunk, (t+1)*chunk)
-  const int chunk = (V + SM_THREADS - 1) / SM_THREADS;
-  const int lo = min(V, t * chunk), hi = min(V, lo + chunk);
   float mine = 0.f;
   for (int i = lo; i < hi; ++i) {
     const float v = x[i];
@@ -182,16 +302,21 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
     found = pick;
   }
   __syncthreads();
-  if (t == 0) out_tokens[r] = found >= 0 ? found : mi;  // rounding left the target past the last token: take the mode
+  if (t == 0) {
+    const int pick = found >= 0 ? found : mi;  // rounding left the target past the last token: take the mode
+    out_tokens[r] = pick;
+    if (mark) mark[pick] = 1;
+  }
 }
 
 TIS_EXPORT int tis_sample(const float* logits, long ld, float* work, int rows, int V, const float* temperature,
                           const int* top_k, const float* top_p, const float* rep_penalty, const int* ctx_tokens,
-                          const int* ctx_offsets, const float* uniform, int* out_tokens, hipStream_t stream) {
+                          const int* ctx_offsets, const float* uniform, int* out_tokens, unsigned char* seen,
+                          long seen_ld, const int* seen_row, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || V < 1) return tis_fail("sample: bad size rows=%d vocab=%d", rows, V);
   sample_kernel<<<rows, SM_THREADS, 0, stream>>>(logits, ld, work, V, temperature, top_k, top_p, rep_penalty,
-                                                 ctx_tokens, ctx_offsets, uniform, out_tokens);
+                                                 ctx_tokens, ctx_offsets, uniform, out_tokens, seen, seen_ld, seen_row);
   return tis_launch_status("sample");
 }
 

@@ -75,7 +75,7 @@ class Scheduler:
         self.max_context = min(max_context or engine.spec.max_context, engine.spec.max_context)
         self.eos = engine.spec.eos_token_id
         self.page_size = engine.page_size
-        self.sampler = Sampler(engine.ops)
+        self.sampler = Sampler(engine.ops, engine.spec.vocab_size, engine.cache.max_requests)
         self.queue: Deque[Request] = deque()
         self.active: List[Request] = []
         self.finished: List[Request] = []
@@ -179,7 +179,9 @@ class Scheduler:
             r.fed += n
         if sampled:
             toks = self.sampler.sample(out.logits, [r.params for r in sampled],
-                                       [len(r.out_ids()) for r in sampled], [r.ids for r in sampled])
+                                       [len(r.out_ids()) for r in sampled], [r.ids for r in sampled],
+                                       slots=[self.engine.requests[r.id][0] for r in sampled],
+                                       owners=[(r.id, r.preempted) for r in sampled])
             for r, t in zip(sampled, toks):
                 r.ids.append(int(t))
                 self.finish_check(r)

@@ -69,7 +69,7 @@ _SIGNATURES = {
         "tis_gemm_plain": [_I, _I, _P, _L, _P, _L, _P, _L, _P, _L, _I, _I, _I, _P],
     }),
     "sampling": ("tis_sampling", {
-        "tis_sample": [_P, _L, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P],
+        "tis_sample": [_P, _L, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P],
         "tis_argmax": [_P, _L, _I, _I, _P, _P],
     }),
 }
@@ -507,8 +507,14 @@ class HipOps:
         self.sampling.tis_argmax(_ptr(logits), logits.stride(0), n, V, _ptr(out), self._stream())
         return out
 
-    def sample(self, logits, temperature, top_k, top_p, rep_penalty, uniform, ctx_tokens=None, ctx_offsets=None):
-        """One token per row of 32-bit logits; per-row parameters are device tensors of length rows."""
+    def sample(self, logits, temperature, top_k, top_p, rep_penalty, uniform, ctx_tokens=None, ctx_offsets=None,
+               seen=None, seen_row=None):
+        """One token per row of 32-bit logits; per-row parameters are device tensors of length rows.
+
+        A request's context for the repetition penalty comes as a flat token list with offsets, or as `seen`, a
+        [requests, vocab] byte table (nonzero: occurred) with `seen_row[i]` naming row i's line (-1: none); the
+        kernel then also marks the token it draws.
+        """
         _rows_view(self._check(logits, "logits", torch.float32), "logits")
         n, V = logits.shape
         for t, what, dt in ((temperature, "temperature", torch.float32), (top_p, "top_p", torch.float32),
@@ -523,9 +529,15 @@ class HipOps:
         if ctx_tokens is not None:
             self._index(ctx_tokens, "ctx_tokens")
             self._index(ctx_offsets, "ctx_offsets", n + 1)
+        if seen is not None:
+            self._check(seen, "seen", torch.uint8)
+            if seen.dim() != 2 or seen.shape[1] != V or seen.stride(1) != 1:
+                raise KernelError(f"sample: seen {tuple(seen.shape)} is not [requests, {V}]")
+            self._index(seen_row, "seen_row", n)
         work = torch.empty(n, V, dtype=torch.float32, device=self.device)
         out = torch.empty(n, dtype=torch.int32, device=self.device)
         self.sampling.tis_sample(_ptr(logits), logits.stride(0), _ptr(work), n, V, _ptr(temperature), _ptr(top_k),
                                  _ptr(top_p), _ptr(rep_penalty), _ptr(ctx_tokens), _ptr(ctx_offsets), _ptr(uniform),
-                                 _ptr(out), self._stream())
+                                 _ptr(out), _ptr(seen), seen.stride(0) if seen is not None else 0,
+                                 _ptr(seen_row if seen is not None else None), self._stream())
         return out

@@ -64,6 +64,8 @@ def main() -> int:
     ap.add_argument("--trunk-only", action="store_true", help="leave the prediction heads out, as the reference's plain decode does")
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure, comma separated ('' for none)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--no-trunk-point", dest="trunk_point", action="store_false",
+                    help="skip the extra decode measurement without the prediction heads")
     ap.add_argument("--seed", type=int, default=0)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -82,9 +84,7 @@ def main() -> int:
     cfg = cfg_full
     if a.layers and a.layers != cfg_full.n_layers:
         cfg = dataclasses.replace(cfg_full, n_layers=a.layers)
-    if a.trunk_only:
-        cfg = dataclasses.replace(cfg, mtp_heads=0)
-    heads = cfg.mtp_heads > 0
+    heads = cfg.mtp_heads > 0 and not a.trunk_only
     dev = "cuda:0"
     torch.cuda.set_device(0)
     tensors = random_tensors(cfg, a.seed, dtype=a.dtype, device=dev)
@@ -92,12 +92,16 @@ def main() -> int:
     max_b = max([a.batch] + points)
     page = 16
     engine = Engine(config=cfg, tensors=tensors, dtype=a.dtype, page_size=page,
-                    max_tokens=max_b * (a.context + page), max_requests=max_b, device=dev)
+                    max_tokens=max_b * (a.context + page), max_requests=max_b, device=dev, run_heads=heads)
+    trunk = None
+    if heads and a.trunk_point:
+        trunk = Engine(config=cfg, tensors=tensors, dtype=a.dtype, page_size=page,
+                       max_tokens=a.batch * (a.context + page), max_requests=a.batch, device=dev, run_heads=False)
     del tensors
     vocab = cfg.vocab_size
     gen = torch.Generator().manual_seed(a.seed)
 
-    def decode_rate(B: int, steps: int, warmup: int):
+    def decode_rate(B: int, steps: int, warmup: int, engine=engine):
         """Tokens a second and seconds per step of `steps` decode steps at batch B near the context length."""
         start_len = a.context - steps - warmup - 1
         rids = [f"b{B}_{i}" for i in range(B)]
@@ -148,6 +152,9 @@ def main() -> int:
     pts = {}
     for B in points:
         pts[f"decode_b{B}"] = round(decode_rate(B, max(8, a.steps // 2), max(2, a.warmup // 2))[0], 1)
+    if trunk is not None:
+        # the reference's "plain" decode runs no prediction heads; the same here, for comparison with its numbers
+        pts[f"decode_b{a.batch}_trunk_only"] = round(decode_rate(a.batch, a.steps, a.warmup, trunk)[0], 1)
     line = {
         "metric": "decode tok/s at batch 8 (0.9B, bf16); prefill tok/s at 2,048 tokens",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -158,7 +165,8 @@ def main() -> int:
             "model": a.size, "global_batch": a.batch, "seq_len": a.context, "parallelism": "single-gpu",
             "n_layers": cfg.n_layers, "n_layers_full": cfg_full.n_layers, "d_model": cfg.d_model,
             "n_heads": cfg.n_heads, "n_kv_heads": cfg.n_kv_heads, "head_dim": cfg.head_dim,
-            "ffn_hidden": cfg.ffn_hidden, "vocab_size": cfg.vocab_size, "mtp_heads_run": cfg.mtp_heads,
+            "ffn_hidden": cfg.ffn_hidden, "vocab_size": cfg.vocab_size,
+            "mtp_heads_run": cfg.mtp_heads if heads else 0,
             "tie_embeddings": cfg.tie_embeddings, "rope_base": cfg.rope_base, "page_size": page,
             "sampling": "greedy",
         },

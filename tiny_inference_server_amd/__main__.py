@@ -64,6 +64,8 @@ def main(argv=None) -> int:
     ap.add_argument("--tokens-per-block", type=int, default=16)
     ap.add_argument("--token-budget", type=int, default=2048, help="most tokens one step runs")
     ap.add_argument("--plan", choices=["final", "cur"], default="final")
+    ap.add_argument("--heads", action="store_true",
+                    help="also run the multi-token-prediction heads at every step (their drafts are not used)")
     a = ap.parse_args(argv)
 
     from .config import load_config
@@ -90,11 +92,11 @@ def main(argv=None) -> int:
         prompts = [[rng.randrange(cfg.vocab_size) for _ in range(a.prompt_len)] for _ in range(a.num_prompts)]
 
     elem = 2 if a.dtype == "bfloat16" else 4
-    planes = cfg.n_layers + cfg.mtp_heads
+    planes = cfg.n_layers + (cfg.mtp_heads if a.heads else 0)
     page_bytes = a.tokens_per_block * 2 * cfg.n_kv_heads * cfg.head_dim * planes * elem      # block_table.py:34-38
     n_pages = max(1, parse_bytes(a.pool_bytes) // page_bytes)
     engine = Engine(model_dir, dtype=a.dtype, page_size=a.tokens_per_block, n_pages=n_pages,
-                    max_requests=a.max_batch, device=a.device)
+                    max_requests=a.max_batch, device=a.device, run_heads=a.heads)
     print(f"POOL: {n_pages} blocks of {a.tokens_per_block} tokens", file=sys.stderr)
     import torch
     t0 = time.time()

@@ -6,6 +6,7 @@ and returns 32-bit logits at the places asked for.
 """
 from __future__ import annotations
 
+import dataclasses
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -39,7 +40,8 @@ class StepOutput:
 class Engine:
     def __init__(self, model_dir: Optional[str] = None, *, config=None, tensors=None, dtype="bfloat16",
                  page_size: int = 16, max_tokens: Optional[int] = None, n_pages: Optional[int] = None,
-                 max_requests: int = 64, device="cuda:0", ops=None, use_graphs: bool = True):
+                 max_requests: int = 64, device="cuda:0", ops=None, use_graphs: bool = True,
+                 run_heads: bool = True):
         self.dtype = resolve_dtype(dtype)
         if model_dir is not None:
             config = load_config(model_dir)
@@ -57,7 +59,10 @@ class Engine:
             ops = HipOps(device, self.dtype)
         self.ops = ops
         self.device = ops.device
-        self.model = Model(self.spec, tensors, ops)
+        # run_heads=False runs the first stage only, as the reference does with spec=False (server.py:118): the
+        # prediction heads' weights are still loaded and checked, but they take no time and no cache
+        self.run_spec = self.spec if run_heads else dataclasses.replace(self.spec, stages=self.spec.stages[:1])
+        self.model = Model(self.run_spec, tensors, ops)
         if n_pages is None:
             if max_tokens is None:
                 raise ValueError("give the cache's size as max_tokens or n_pages")

@@ -39,12 +39,15 @@ static constexpr int DB = HD / 16;          // 16-wide blocks of the head for P.
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x4 load4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
 
-template <int NB>
+// PS16: pages of exactly 16 tokens. A 16-key tile is then a whole page, page indices are shifts, and a lane's
+// offsets inside a page never change: the loads of a step need no address arithmetic beyond the page's base.
+template <int NB, bool PS16>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 : 1))) void attention_mfma_kernel(
     const bf16* __restrict__ q, long q_ld, const bf16* __restrict__ plane, const int* __restrict__ block_tables,
     int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ items,
     bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
-    int n_kv_heads, int n_heads, int page_size, int window, float scale_log2, int n_splits) {
+    int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits) {
+  const int page_size = PS16 ? 16 : page_size_arg;
   const int item = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int lane = threadIdx.x, c16 = lane & 15, g = lane >> 4;
   const int row0 = items[item].x, n_rows = items[item].y;
@@ -118,7 +121,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     for (int t = 0; t < 2; ++t) {
       const int key0 = k_lo + s * 32 + t * 16;
       const bool ok = s < s_end && key0 < k_hi;
-      const int got = bt[ok ? key0 / page_size : 0];
+      const int got = bt[ok ? (PS16 ? key0 >> 4 : key0 / page_size) : 0];
       pg[t] = ok ? got : -1;
     }
   };
@@ -126,7 +129,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int key0 = k_lo + s * 32 + t * 16;
-      const int slot0 = key0 % page_size;
+      const int slot0 = PS16 ? 0 : key0 % page_size;
       T.ok[t] = pg[t] >= 0;
       const bf16* base = plane + (long)(T.ok[t] ? pg[t] : 0) * page_stride;
       const bf16* kp = base + k_head + (long)(slot0 + c16) * HD;
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          float v = st[t][nb][i] * scale_log2;
+          float v = st[t][nb][i];         // unscaled: the scale (positive) goes into the exponent's multiply-add
           if (!full) {
             const int key = kb + t * 16 + g * 4 + i;
             const bool ok = T.ok[t] && key <= col_pos[nb] && key >= col_lo[nb];
@@ -185,6 +188,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
         }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      tmax *= scale_log2;
       // m is the exponent that P, the sum and the output are taken relative to. It follows the running maximum
       // only when that has grown by more than 2^8 beyond it, so it settles after a row's first keys and the
       // rescaling below becomes rare; until then P stays below 256, well inside bfloat16, and sum and output
@@ -198,7 +202,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
       bf16x8 pv;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = __builtin_amdgcn_exp2f(sv[e] - m_use);   // arguments are <= 8: no overflow to guard
+        const float p = __builtin_amdgcn_exp2f(fmaf(sv[e], scale_log2, -m_use));   // arguments are <= 8
         psum += p;
         pv[e] = static_cast<__bf16>(p);
       }
@@ -358,14 +362,20 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
     return tis_fail("attention_mfma: q, out and the cache plane must be 16-byte aligned with row strides in steps of 8");
   dim3 grid(n_items, n_kv_heads, n_splits);
   const float scale_log2 = scale * 1.4426950408889634f;
-#define LAUNCH(NBV)                                                                                              \
-  attention_mfma_kernel<NBV><<<grid, 64, 0, stream>>>(                                                           \
+#define LAUNCH(NBV, PSV)                                                                                              \
+  attention_mfma_kernel<NBV, PSV><<<grid, 64, 0, stream>>>(                                                      \
       (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)items,     \
       (bf16*)out, out_ld, part_o, (float2*)part_ml, group, n_kv_heads, n_heads, page_size, window, scale_log2,   \
       n_splits)
-  if (nb == 1) LAUNCH(1);
-  else if (nb == 2) LAUNCH(2);
-  else LAUNCH(4);
+  if (page_size == 16) {
+    if (nb == 1) LAUNCH(1, true);
+    else if (nb == 2) LAUNCH(2, true);
+    else LAUNCH(4, true);
+  } else {
+    if (nb == 1) LAUNCH(1, false);
+    else if (nb == 2) LAUNCH(2, false);
+    else LAUNCH(4, false);
+  }
 #undef LAUNCH
   int rc = tis_launch_status("attention_mfma");
   if (rc) return rc;

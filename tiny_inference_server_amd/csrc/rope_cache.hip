@@ -15,60 +15,64 @@
 
 TIS_DEFINE_LAST_ERROR(tis_rope_cache)
 
-template <typename T>
-__global__ __launch_bounds__(64) void rope_write_kv_kernel(T* __restrict__ qkv, long ld, const int* __restrict__ positions,
-                                                           const int* __restrict__ write_slots,
-                                                           const float2* __restrict__ table, T* __restrict__ plane,
-                                                           int n_heads, int n_kv_heads, int head_dim, int page_size,
-                                                           int interleaved, int write_cache, int paired,
-                                                           T* __restrict__ q_out, long q_out_ld) {
-  const long r = blockIdx.x;
-  const int hh = blockIdx.y;  // [0, n_heads): q, then k heads, then v heads
-  const int half = head_dim / 2;
-  T* row = qkv + r * ld + (long)hh * head_dim;
+static constexpr int RC_THREADS = 256;
 
-  T* dst = row;  // queries are rewritten where they are, unless a separate output is given
-  const bool is_q = hh < n_heads;
-  if (is_q && q_out) dst = q_out + r * q_out_ld + (long)hh * head_dim;
-  const bool is_v = hh >= n_heads + n_kv_heads;
-  if (!is_q) {
-    if (!write_cache) {
-      return;  // keys and values that are not kept have no reader
-    } else {
-      const int slot = write_slots[r];
-      const int page = slot / page_size, off = slot % page_size;
+// One workgroup per row; its four waves take the row's heads (q, then k, then v) in turn.
+template <typename T>
+__global__ __launch_bounds__(RC_THREADS) void rope_write_kv_kernel(T* __restrict__ qkv, long ld,
+                                                                   const int* __restrict__ positions,
+                                                                   const int* __restrict__ write_slots,
+                                                                   const float2* __restrict__ table,
+                                                                   T* __restrict__ plane, int n_heads, int n_kv_heads,
+                                                                   int head_dim, int page_size, int interleaved,
+                                                                   int write_cache, int paired, T* __restrict__ q_out,
+                                                                   long q_out_ld) {
+  const long r = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int half = head_dim / 2;
+  const int total = n_heads + 2 * n_kv_heads;
+  const int slot = write_cache ? write_slots[r] : 0;
+  const int page = slot / page_size, off = slot % page_size;
+  const float2* cs = table ? table + (long)positions[r] * half : nullptr;
+
+  for (int hh = threadIdx.x >> 6; hh < total; hh += RC_THREADS / 64) {   // [0, n_heads): q, then k heads, then v heads
+    T* row = qkv + r * ld + (long)hh * head_dim;
+    const bool is_q = hh < n_heads;
+    const bool is_v = hh >= n_heads + n_kv_heads;
+    T* dst = row;  // queries are rewritten where they are, unless a separate output is given
+    if (is_q && q_out) dst = q_out + r * q_out_ld + (long)hh * head_dim;
+    if (!is_q) {
+      if (!write_cache) continue;  // keys and values that are not kept have no reader
       const int kvh = is_v ? hh - n_heads - n_kv_heads : hh - n_heads;
       T* head = plane + (((long)page * 2 + (is_v ? 1 : 0)) * n_kv_heads + kvh) * page_size * head_dim;
       if (is_v) {  // values: [head_dim][slot]
-        for (int i = threadIdx.x; i < head_dim; i += blockDim.x) head[(long)i * page_size + off] = row[i];
-        return;
+        for (int i = lane; i < head_dim; i += 64) head[(long)i * page_size + off] = row[i];
+        continue;
       }
       dst = head + (long)off * head_dim;
     }
-  }
-  if (is_v) return;
-  if (table == nullptr) {
-    if (paired) {
-      for (int j = threadIdx.x; j < half; j += blockDim.x) {
-        dst[interleaved ? 2 * j : j] = row[2 * j];
-        dst[interleaved ? 2 * j + 1 : j + half] = row[2 * j + 1];
+    if (cs == nullptr) {
+      if (paired) {
+        for (int j = lane; j < half; j += 64) {
+          dst[interleaved ? 2 * j : j] = row[2 * j];
+          dst[interleaved ? 2 * j + 1 : j + half] = row[2 * j + 1];
+        }
+      } else if (dst != row) {
+        for (int i = lane; i < head_dim; i += 64) dst[i] = row[i];
       }
-    } else if (dst != row) {
-      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = row[i];
+      continue;
     }
-    return;
-  }
-  const float2* cs = table + (long)positions[r] * half;
-  for (int j = threadIdx.x; j < half; j += blockDim.x) {
-    const int a = interleaved ? 2 * j : j;
-    const int b = interleaved ? 2 * j + 1 : j + half;
-    const float x1 = to_f(row[paired ? 2 * j : a]), x2 = to_f(row[paired ? 2 * j + 1 : b]);
-    const float c = cs[j].x, s = cs[j].y;
-    // q*cos + rotate_half(q)*sin with rotate_half = [-x2, x1]
-    const float y1 = x1 * c - x2 * s;
-    const float y2 = x2 * c + x1 * s;
-    dst[a] = from_f<T>(y1);
-    dst[b] = from_f<T>(y2);
+    for (int j = lane; j < half; j += 64) {
+      const int a = interleaved ? 2 * j : j;
+      const int b = interleaved ? 2 * j + 1 : j + half;
+      const float x1 = to_f(row[paired ? 2 * j : a]), x2 = to_f(row[paired ? 2 * j + 1 : b]);
+      const float c = cs[j].x, s = cs[j].y;
+      // q*cos + rotate_half(q)*sin with rotate_half = [-x2, x1]
+      const float y1 = x1 * c - x2 * s;
+      const float y2 = x2 * c + x1 * s;
+      dst[a] = from_f<T>(y1);
+      dst[b] = from_f<T>(y2);
+    }
   }
 }
 
@@ -80,15 +84,14 @@ TIS_EXPORT int tis_rope_write_kv(int dtype, void* qkv, long ld, const int* posit
   if (rows < 0 || n_heads < 1 || n_kv_heads < 1 || head_dim < 2 || (head_dim & 1) || page_size < 1)
     return tis_fail("rope_write_kv: bad size rows=%d heads=%d kv_heads=%d head_dim=%d page=%d", rows, n_heads,
                     n_kv_heads, head_dim, page_size);
-  if (n_heads + 2 * n_kv_heads > 65535) return tis_fail("rope_write_kv: too many heads for the grid");
   if (paired && !q_out) return tis_fail("rope_write_kv: paired input needs a separate output for the queries");
-  dim3 grid(rows, n_heads + 2 * n_kv_heads);
+  dim3 grid(rows);
   if (dtype == TIS_F32)
-    rope_write_kv_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, ld, positions, write_slots, (const float2*)table,
+    rope_write_kv_kernel<float><<<grid, RC_THREADS, 0, stream>>>((float*)qkv, ld, positions, write_slots, (const float2*)table,
                                                          (float*)plane, n_heads, n_kv_heads, head_dim, page_size,
                                                          interleaved, write_cache, paired, (float*)q_out, q_out_ld);
   else if (dtype == TIS_BF16)
-    rope_write_kv_kernel<bf16><<<grid, 64, 0, stream>>>((bf16*)qkv, ld, positions, write_slots, (const float2*)table,
+    rope_write_kv_kernel<bf16><<<grid, RC_THREADS, 0, stream>>>((bf16*)qkv, ld, positions, write_slots, (const float2*)table,
                                                         (bf16*)plane, n_heads, n_kv_heads, head_dim, page_size,
                                                         interleaved, write_cache, paired, (bf16*)q_out, q_out_ld);
   else

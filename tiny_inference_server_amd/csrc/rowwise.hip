@@ -29,6 +29,49 @@ __global__ __launch_bounds__(ROW_THREADS) void rmsnorm_kernel(const T* x, long x
   rmsnorm_row<T>(x + r * x_ld, gain, y + r * y_ld, D, eps, scratch);
 }
 
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+
+// The same norm for bfloat16 rows whose width is a multiple of 8 and whose rows start on 16 bytes: every thread
+// moves 16 bytes at a time and keeps its values in registers between the two passes.
+template <int PER_THREAD>
+__global__ __launch_bounds__(ROW_THREADS) void rmsnorm_bf16_vec_kernel(const bf16* __restrict__ x, long x_ld,
+                                                                       const float* __restrict__ gain,
+                                                                       bf16* __restrict__ y, long y_ld, int D,
+                                                                       float eps) {
+  __shared__ float scratch[16];
+  const long r = blockIdx.x;
+  const bf16* xr = x + r * x_ld;
+  bf16* yr = y + r * y_ld;
+  bf16x8 v[PER_THREAD];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER_THREAD; ++i) {
+    const int c = (i * ROW_THREADS + threadIdx.x) * 8;
+    if (c < D) {
+      v[i] = *reinterpret_cast<const bf16x8*>(xr + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = static_cast<float>(v[i][e]);
+        ss += f * f;
+      }
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float mul = sqrtf((float)D) / (sqrtf(ss) + eps);
+#pragma unroll
+  for (int i = 0; i < PER_THREAD; ++i) {
+    const int c = (i * ROW_THREADS + threadIdx.x) * 8;
+    if (c < D) {
+      const float4 g0 = *reinterpret_cast<const float4*>(gain + c), g1 = *reinterpret_cast<const float4*>(gain + c + 4);
+      const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+      bf16x8 w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) w[e] = static_cast<__bf16>(static_cast<float>(v[i][e]) * mul * g[e]);
+      *reinterpret_cast<bf16x8*>(yr + c) = w;
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(ROW_THREADS) void embedding_kernel(const T* table, const int* tokens, T* out,
                                                                 long out_ld, int D) {
@@ -67,6 +110,25 @@ __global__ __launch_bounds__(ROW_THREADS) void copy_rows_kernel(const T* src, lo
   for (int c = threadIdx.x; c < D; c += blockDim.x) to[c] = from[c];
 }
 
+// The gate for bfloat16 rows of a width that is a multiple of 8, 16-byte aligned: eight outputs per thread.
+__global__ __launch_bounds__(ROW_THREADS) void swiglu_bf16_vec_kernel(const bf16* __restrict__ gu, long gu_ld,
+                                                                      bf16* __restrict__ out, long out_ld, int F) {
+  const long r = blockIdx.x;
+  const int f = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (f >= F) return;
+  const bf16x8 a = *reinterpret_cast<const bf16x8*>(gu + r * gu_ld + 2 * f);
+  const bf16x8 b = *reinterpret_cast<const bf16x8*>(gu + r * gu_ld + 2 * f + 8);
+  bf16x8 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float g0 = static_cast<float>(a[2 * e]), u0 = static_cast<float>(a[2 * e + 1]);
+    const float g1 = static_cast<float>(b[2 * e]), u1 = static_cast<float>(b[2 * e + 1]);
+    o[e] = static_cast<__bf16>(g0 / (1.f + expf(-g0)) * u0);
+    o[4 + e] = static_cast<__bf16>(g1 / (1.f + expf(-g1)) * u1);
+  }
+  *reinterpret_cast<bf16x8*>(out + r * out_ld + f) = o;
+}
+
 // out[r, f] = silu(gu[r, 2f]) * gu[r, 2f + 1]: gate and up columns come interleaved  (reference main_models_new.py:51)
 template <typename T>
 __global__ __launch_bounds__(ROW_THREADS) void swiglu_kernel(const T* gu, long gu_ld, T* out, long out_ld, int F) {
@@ -87,6 +149,17 @@ TIS_EXPORT int tis_rmsnorm(int dtype, const void* x, long x_ld, const float* gai
                            int D, float eps, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || D < 1) return tis_fail("rmsnorm: bad size rows=%d D=%d", rows, D);
+  if (dtype == TIS_BF16 && D % 8 == 0 && D <= 8 * 8 * ROW_THREADS && x_ld % 8 == 0 && y_ld % 8 == 0 &&
+      (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0 && (uintptr_t)gain % 16 == 0) {
+    const int per_thread = (D / 8 + ROW_THREADS - 1) / ROW_THREADS;
+#define VEC(P) rmsnorm_bf16_vec_kernel<P><<<rows, ROW_THREADS, 0, stream>>>((const bf16*)x, x_ld, gain, (bf16*)y, y_ld, D, eps)
+    if (per_thread <= 1) VEC(1);
+    else if (per_thread <= 2) VEC(2);
+    else if (per_thread <= 4) VEC(4);
+    else VEC(8);
+#undef VEC
+    return tis_launch_status("rmsnorm");
+  }
   DISPATCH(dtype, (rmsnorm_kernel<T><<<rows, ROW_THREADS, 0, stream>>>((const T*)x, x_ld, gain, (T*)y, y_ld, D, eps)))
   return tis_launch_status("rmsnorm");
 }
@@ -131,6 +204,12 @@ TIS_EXPORT int tis_swiglu(int dtype, const void* gu, long gu_ld, void* out, long
   if (rows == 0) return 0;
   if (rows < 0 || F < 1) return tis_fail("swiglu: bad size rows=%d F=%d", rows, F);
   if ((F + ROW_THREADS - 1) / ROW_THREADS > 65535) return tis_fail("swiglu: width %d exceeds the grid", F);
+  if (dtype == TIS_BF16 && F % 8 == 0 && gu_ld % 8 == 0 && out_ld % 8 == 0 && (uintptr_t)gu % 16 == 0 &&
+      (uintptr_t)out % 16 == 0) {
+    dim3 vgrid(rows, (F / 8 + ROW_THREADS - 1) / ROW_THREADS);
+    swiglu_bf16_vec_kernel<<<vgrid, ROW_THREADS, 0, stream>>>((const bf16*)gu, gu_ld, (bf16*)out, out_ld, F);
+    return tis_launch_status("swiglu");
+  }
   dim3 grid(rows, (F + ROW_THREADS - 1) / ROW_THREADS);
   DISPATCH(dtype, (swiglu_kernel<T><<<grid, ROW_THREADS, 0, stream>>>((const T*)gu, gu_ld, (T*)out, out_ld, F)))
   return tis_launch_status("swiglu");

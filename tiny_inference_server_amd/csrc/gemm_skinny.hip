@@ -1,7 +1,7 @@
 // C[M,N] = f(A[M,K]) . W[N,K]^T for few rows (M <= 16): the matrix product of decode steps, where the job is to
 // stream W from HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950).
 //
-// One workgroup owns 16 rows of W (16 output columns) over the whole of K; its waves take the 32-wide steps of
+// One workgroup owns 16 rows of W (16 output columns; 8 in the narrow variant below) over the whole of K; its waves take the 32-wide steps of
 // K in turn, so together they read each weight row in contiguous runs. W rows are the A operand straight from
 // global memory (16 bytes per lane), the activations are the B operand straight from L2 (they are a few KB
 // and every workgroup reads the same ones), so no LDS is used for operands. Partial sums of the waves are
@@ -43,114 +43,112 @@ struct RopeArgs {
 // GS_WAVES: waves per workgroup; U: steps of K whose loads a wave issues together before the first product.
 // Eight waves of three or four steps measured best on MI355X for K of 1536 to 4096 (5.6 us for a 25 MB matrix,
 // 23 us for the 147 MB output table: 80 % of the HBM peak); four waves where K is too short to feed eight.
-template <int MB, bool NORM, int EPI, typename TO, int GS_WAVES, int U>
+//
+// R: with 16 output columns per workgroup a matrix of 1536 rows gives 96 workgroups, and a compute unit draws
+// only about 24 GB/s, so the 160 idle units cost more than the product. For M <= 16/R rows a workgroup
+// therefore owns only 16/R columns and fills the 16 rows of the matrix operand with R different 32-wide chunks of
+// K for those columns; the activation operand holds the same R chunks side by side. Of the 16x16 result only
+// the R diagonal blocks (chunk r of the weights against chunk r of the activations) mean anything; they are
+// added up with the waves' partial sums. R times as many workgroups, each step covers 32 R of K.
+template <bool NORM, int EPI, typename TO, int GS_WAVES, int U, int R>
 __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
     const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const float* __restrict__ gain, float eps,
-    const bf16* __restrict__ R, long r_ld, TO* __restrict__ C, long c_ld, int M, int N, int K, RopeArgs rope) {
-  __shared__ float red[GS_WAVES][MB][64][4];
-  __shared__ float red_ss[GS_WAVES][MB][16];
+    const bf16* __restrict__ R_in, long r_ld, TO* __restrict__ C, long c_ld, int M, int N, int K, RopeArgs rope) {
+  constexpr int COLS = 16 / R;   // output columns of a workgroup, and the most rows of X it takes
+  constexpr int GH = 4 / R;      // lane groups of four result rows per chunk
+  __shared__ float red[GS_WAVES][64][4];
+  __shared__ float red_ss[GS_WAVES][16];
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const int steps = (K + 31) / 32;
-  const bool w_ok = n0 + c16 < N;
-  const bf16* wrow = W + (long)(n0 + c16) * K + g * 8;
+  const int chunk = c16 / COLS, sub = c16 % COLS;   // the lane's chunk of a step; its weight row and its activation row
+  const int n0 = blockIdx.x * COLS;
+  const int steps = (K + 32 * R - 1) / (32 * R);
+  const bool w_ok = n0 + sub < N;
+  const bool x_ok = sub < M;
+  const bf16* wrow = W + (long)(w_ok ? n0 + sub : 0) * K + chunk * 32 + g * 8;
+  const bf16* xrow = X + (long)(x_ok ? sub : 0) * x_ld + chunk * 32 + g * 8;
 
-  f32x4 acc[MB];
-  float ss[MB];
-  const bf16* xrow[MB];
-  bool x_ok[MB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    acc[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    ss[mb] = 0.f;
-    const int m = mb * 16 + c16;
-    x_ok[mb] = m < M;
-    xrow[mb] = X + (long)(x_ok[mb] ? m : 0) * x_ld + g * 8;
-  }
+  f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float ss = 0.f;
 
   // U steps at a time: all their loads are issued before the first product, so that a wave keeps several
   // rows' worth of HBM requests in flight
   for (int s0 = wave; s0 < steps; s0 += U * GS_WAVES) {
     bf16x8 a[U];
-    bf16x8 b[U][MB];
+    bf16x8 b[U];
     float gv[U][8];
-    bool k_ok[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int s = s0 + u * GS_WAVES;
-      const int k = s * 32 + g * 8;
-      k_ok[u] = s < steps && k < K;   // K is a multiple of 8, so a lane's 8 values are all inside or all outside
+      const int k = s * (32 * R) + chunk * 32 + g * 8;
+      const bool k_ok = s < steps && k < K;   // K is a multiple of 8, so a lane's 8 values are all inside or all outside
       a[u] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-      if (w_ok && k_ok[u]) a[u] = *reinterpret_cast<const bf16x8*>(wrow + (long)s * 32);
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        b[u][mb] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-        if (x_ok[mb] && k_ok[u]) b[u][mb] = *reinterpret_cast<const bf16x8*>(xrow[mb] + (long)s * 32);
-      }
+      b[u] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+      if (w_ok && k_ok) a[u] = *reinterpret_cast<const bf16x8*>(wrow + (long)s * (32 * R));
+      if (x_ok && k_ok) b[u] = *reinterpret_cast<const bf16x8*>(xrow + (long)s * (32 * R));
       if (NORM) {
-        const float4 g0 = k_ok[u] ? *reinterpret_cast<const float4*>(gain + k) : make_float4(0.f, 0.f, 0.f, 0.f);
-        const float4 g1 = k_ok[u] ? *reinterpret_cast<const float4*>(gain + k + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 g0 = k_ok ? *reinterpret_cast<const float4*>(gain + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 g1 = k_ok ? *reinterpret_cast<const float4*>(gain + k + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
         gv[u][0] = g0.x; gv[u][1] = g0.y; gv[u][2] = g0.z; gv[u][3] = g0.w;
         gv[u][4] = g1.x; gv[u][5] = g1.y; gv[u][6] = g1.z; gv[u][7] = g1.w;
       }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
+      bf16x8 bv = b[u];
+      if (NORM) {
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        bf16x8 bv = b[u][mb];
-        if (NORM) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float xf = static_cast<float>(bv[e]);
-            ss[mb] += xf * xf;
-            bv[e] = static_cast<__bf16>(xf * gv[u][e]);
-          }
+        for (int e = 0; e < 8; ++e) {
+          const float xf = static_cast<float>(bv[e]);
+          ss += xf * xf;
+          bv[e] = static_cast<__bf16>(xf * gv[u][e]);
         }
-        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc[mb], 0, 0, 0);
       }
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc, 0, 0, 0);
     }
   }
 
-  // add the waves' partial sums in a fixed order
+  // add the partial sums of the waves and of the chunks in a fixed order
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][mb][lane][i] = acc[mb][i];
-    if (NORM) {
-      float t = ss[mb];
-      t += __shfl_xor(t, 16, 64);
-      t += __shfl_xor(t, 32, 64);
-      if (g == 0) red_ss[wave][mb][c16] = t;
-    }
+  for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
+  if (NORM) {
+    float t = ss;
+    t += __shfl_xor(t, 16, 64);
+    t += __shfl_xor(t, 32, 64);
+    if (g == 0) red_ss[wave][c16] = t;
   }
   __syncthreads();
   if (wave != 0) return;
-
+  // result lane (gh, m): columns n0 + 4 gh + i of row m; chunk r's share sits with lane (r GH + gh, r COLS + m)
+  const int gh = lane >> 4, m = lane & 15;
+  if (gh >= GH || m >= COLS || m >= M) return;
+  float v[4];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    const int m = mb * 16 + c16;
-    float v[4];
+  for (int i = 0; i < 4; ++i) {
+    float t = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float t = red[0][mb][lane][i];
+    for (int r = 0; r < R; ++r) {
+      const int src = (r * GH + gh) * 16 + r * COLS + m;
 #pragma unroll
-      for (int w = 1; w < GS_WAVES; ++w) t += red[w][mb][lane][i];
-      v[i] = t;
+      for (int w = 0; w < GS_WAVES; ++w) t += red[w][src][i];
     }
-    if (NORM) {
-      float t = red_ss[0][mb][c16];
+    v[i] = t;
+  }
+  if (NORM) {
+    float t = 0.f;
 #pragma unroll
-      for (int w = 1; w < GS_WAVES; ++w) t += red_ss[w][mb][c16];
-      const float mul = sqrtf((float)K) / (sqrtf(t) + eps);
+    for (int r = 0; r < R; ++r) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] *= mul;
+      for (int w = 0; w < GS_WAVES; ++w) t += red_ss[w][r * COLS + m];
     }
-    if (m >= M) continue;
-    const int n = n0 + g * 4;   // the lane's four consecutive output columns
+    const float mul = sqrtf((float)K) / (sqrtf(t) + eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] *= mul;
+  }
+  {
+    const int n = n0 + gh * 4;   // the lane's four consecutive output columns
     if (EPI == EPI_ROPE) {
-      if (n >= N) continue;          // N is a multiple of head_dim, head_dim of 4: the lane's columns are all in or out
+      if (n >= N) return;          // N is a multiple of head_dim, head_dim of 4: the lane's columns are all in or out
       const int hd = rope.head_dim, half = hd / 2;
       const int head = n / hd, e0 = n % hd;      // e0 is a multiple of 4: two whole pairs
       const bool is_q = head < rope.n_heads, is_v = head >= rope.n_heads + rope.n_kv_heads;
@@ -200,7 +198,7 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
       for (int i = 0; i < 4; ++i) {
         if (n + i < N) {
           float t = v[i];
-          if (EPI == EPI_RESIDUAL) t += static_cast<float>(R[(long)m * r_ld + n + i]);
+          if (EPI == EPI_RESIDUAL) t += static_cast<float>(R_in[(long)m * r_ld + n + i]);
           C[(long)m * c_ld + n + i] = from_f<TO>(t);
         }
       }
@@ -208,28 +206,56 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
   }
 }
 
-template <int MB, bool NORM, int EPI, typename TO>
-static void launch(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
-                   void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope = RopeArgs()) {
-  const int steps = (K + 31) / 32;
-  const int per_wave = (steps + 7) / 8;
-  if (steps >= 24 && per_wave % 3 == 0 && per_wave % 4 != 0)
-    gemm_skinny_kernel<MB, NORM, EPI, TO, 8, 3><<<(N + 15) / 16, 8 * 64, 0, stream>>>(
-        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);
-  else if (steps >= 24)
-    gemm_skinny_kernel<MB, NORM, EPI, TO, 8, 4><<<(N + 15) / 16, 8 * 64, 0, stream>>>(
-        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);
-  else
-    gemm_skinny_kernel<MB, NORM, EPI, TO, 4, 4><<<(N + 15) / 16, 4 * 64, 0, stream>>>(
-        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);
+// A hook for tuning runs: forces (waves, U, R) for every launch of this process; zeros give the choice back.
+static int g_force_waves = 0, g_force_u = 0, g_force_r = 0;
+TIS_EXPORT void tis_gemm_skinny_force_config(int waves, int u, int r) {
+  g_force_waves = waves;
+  g_force_u = u;
+  g_force_r = r;
+}
+
+template <bool NORM, int EPI, typename TO>
+static int launch(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
+                  void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope = RopeArgs()) {
+  // half as wide column tiles where full ones would leave more than half of the 256 compute units idle and the
+  // rows allow it (measured at N = 1536: 6.2 instead of 8.2 us for K = 4096, 4.1 instead of 4.8 us for K = 1536;
+  // at N = 2304 with the norm in front the wider tile stays ahead, and a quarter tile never beat the half)
+  int r = (M <= 8 && (N + 15) / 16 <= 128) ? 2 : 1;
+  if (g_force_r) r = g_force_r;
+  if (r != 1 && r != 2) return tis_fail("gemm_skinny: %d chunks a step; 1 or 2 are built", r);
+  if (M > 16 / r) return tis_fail("gemm_skinny: %d rows do not fit %d columns a workgroup", M, 16 / r);
+  const int steps = (K + 32 * r - 1) / (32 * r);
+  int waves, u;
+  if (steps >= 24) {
+    waves = 8;
+    const int per_wave = (steps + 7) / 8;
+    u = (per_wave % 3 == 0 && per_wave % 4 != 0) ? 3 : 4;
+  } else {
+    waves = 4;
+    u = (steps % 3 == 0 && steps % 4 != 0) || steps == 12 ? 3 : 4;
+  }
+  if (g_force_waves) { waves = g_force_waves; u = g_force_u; }
+  const int cols = 16 / r;
+  const int n_wg = (N + cols - 1) / cols;
+#define CFG(WV, UV, RV)                                                                                          \
+  if (waves == WV && u == UV && r == RV) {                                                                       \
+    gemm_skinny_kernel<NORM, EPI, TO, WV, UV, RV><<<n_wg, WV * 64, 0, stream>>>(                                 \
+        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);     \
+    return 0;                                                                                                    \
+  }
+#define CFGS(RV) CFG(4, 3, RV) CFG(4, 4, RV) CFG(8, 3, RV) CFG(8, 4, RV)
+  CFGS(1) CFGS(2)
+#undef CFGS
+#undef CFG
+  return tis_fail("gemm_skinny: no kernel for %d waves of %d steps and %d chunks", waves, u, r);
 }
 
 template <bool NORM, int EPI, typename TO>
 static int launch_mb(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
                      void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope = RopeArgs()) {
-  // one block of 16 rows: with more rows the library's product is faster than this kernel even after paying for
-  // the separate norm, gating and rotary launches, so more blocks (MB > 1) are not built
-  launch<1, NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
+  // 16 rows at most: with more rows the library's product is faster than this kernel even after paying for
+  // the separate norm, gating and rotary launches
+  if (launch<NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope)) return -1;
   return tis_launch_status("gemm_skinny");
 }
 

@@ -14,6 +14,8 @@ Per stage:
   source_index[r]              for stages that read the previous stage: its row index there, or -(slot+1)
                                for the row kept in the request's state slot
   keep_source[i], keep_slot[i] previous-stage rows to keep in state slots after the reads
+  previous_rows                how many rows read the previous stage's rows of this step; with none, the stage
+                               does not wait for the previous one
   want_index[i]                the rows whose outputs are asked for (-1 where this stage has no such row yet)
 """
 from __future__ import annotations
@@ -49,6 +51,7 @@ class StageBatch:
     keep_source: Optional[torch.Tensor]
     keep_slot: Optional[torch.Tensor]
     keep_count: int
+    previous_rows: int         # rows that read the previous stage's output of this very step (the others: state)
     want_index: torch.Tensor
     want_valid: List[bool]
     max_kv_len: int
@@ -147,35 +150,44 @@ def plan_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: S
 
     plans = []
     prev_rows: Optional[List[Tuple[int, int, int]]] = None
+    entry_tokens = [np.asarray(e.tokens, dtype=np.int64).reshape(-1) for e in entries]
+    empty = np.zeros(0, dtype=np.int64)
+
+    def joined(parts):
+        return np.concatenate(parts) if parts else empty
+
     for j, lag in enumerate(lags):
         tokens, positions, row_seq, cu = [], [], [], [0]
         seq_rows = []
         source, keep_src, keep_slot = [], [], []
+        n_rows = 0
         for k, e in enumerate(entries):
             s, n_tok = e.start, len(e.tokens)
             end = s + n_tok
             p0 = max(0, s - lag)
             n = max(0, end - lag - p0)
-            off = len(e.tokens) - n
-            first_row = len(tokens)
+            first_row = n_rows
             if end > max_context:
                 raise ValueError(f"request in slot {e.slot} would reach position {end - 1}, "
                                  f"beyond the model's context of {max_context}")
-            tokens.extend(int(t) for t in e.tokens[off:])
-            positions.extend(range(p0, p0 + n))
-            row_seq.extend([k] * n)
-            cu.append(len(tokens))
+            pos = np.arange(p0, p0 + n, dtype=np.int64)
+            tokens.append(entry_tokens[k][n_tok - n:])
+            positions.append(pos)
+            row_seq.append(np.full(n, k, dtype=np.int64))
+            n_rows += n
+            cu.append(n_rows)
             seq_rows.append((first_row, p0, n))
             if has_source[j]:
                 pfirst, pp0, pn = prev_rows[k]
-                for p in range(p0, p0 + n):
-                    source.append(pfirst + (p - pp0) if p >= pp0 else -(e.slot + 1))
+                # a row reads the previous stage's row at its position, or the request's kept row before the portion
+                source.append(np.where(pos >= pp0, pfirst + (pos - pp0), -(e.slot + 1)))
                 if pn > 0:
                     keep_src.append(pfirst + pn - 1)
                     keep_slot.append(e.slot)
+        tokens, positions, row_seq, source = joined(tokens), joined(positions), joined(row_seq), joined(source)
         ws = {}
         for gname, g in cache.groups.items():
-            arr = np.empty(len(tokens), dtype=np.int32)
+            arr = np.empty(n_rows, dtype=np.int32)
             for k, e in enumerate(entries):
                 first_row, p0, n = seq_rows[k]
                 if n:
@@ -195,12 +207,13 @@ def plan_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: S
                 valid.append(ok)
         extra = plan_rows(seq_rows, pk.add) if plan_rows is not None else {}
         plans.append(dict(
-            extra=extra, lag=lag, n_rows=len(tokens), tokens=pk.add(tokens), positions=pk.add(positions),
+            extra=extra, lag=lag, n_rows=n_rows, tokens=pk.add(tokens), positions=pk.add(positions),
             row_seq=pk.add(row_seq), cu=pk.add(cu), ws=ws,
             source=pk.add(source) if has_source[j] else None,
             keep_src=pk.add(keep_src) if has_source[j] else None,
             keep_slot=pk.add(keep_slot) if has_source[j] else None,
-            keep_count=len(keep_src), want=pk.add(want), valid=valid, seq_rows=seq_rows,
+            keep_count=len(keep_src), previous_rows=int((source >= 0).sum()) if has_source[j] else 0,
+            want=pk.add(want), valid=valid, seq_rows=seq_rows,
             max_kv=max([p0 + n for _, p0, n in seq_rows if n > 0] or [0]),
             max_rows=max([n for _, _, n in seq_rows] or [0])))
         prev_rows = seq_rows
@@ -224,7 +237,7 @@ def materialize(plan: StepPlan, device, host: Optional[torch.Tensor] = None,
             source_index=dev[pl["source"]] if pl["source"] is not None else None,
             keep_source=dev[pl["keep_src"]] if pl["keep_src"] is not None else None,
             keep_slot=dev[pl["keep_slot"]] if pl["keep_slot"] is not None else None,
-            keep_count=pl["keep_count"], want_index=dev[pl["want"]], want_valid=pl["valid"],
+            keep_count=pl["keep_count"], previous_rows=pl["previous_rows"], want_index=dev[pl["want"]], want_valid=pl["valid"],
             max_kv_len=pl["max_kv"], max_seq_rows=pl["max_rows"], seq_rows=pl["seq_rows"],
             host_slots=[e.slot for e in entries],
             extras={k: (dev[v[0]],) + tuple(v[1:]) for k, v in pl["extra"].items()}))

@@ -67,30 +67,43 @@ class Model:
     def cache_needs(self) -> Dict[str, object]:
         return dict(self.needs)
 
+    def _run_stage(self, j, step, cache, prev):
+        st, b = self.spec.stages[j], step.stages[j]
+        state = cache.states.get(self.state_keys[j]) if self.state_keys[j] else None
+        x = self.inputs[j].forward(b, prev, self.shared, state)
+        if b.n_rows:
+            for i, call in enumerate(st.calls):
+                key = self.call_keys[j][i]
+                need = self.needs.get(key)
+                # the rows going into a layer are replaced by its result: the layer may overwrite them
+                ctx = CallContext(batch=b, writes_cache=call.writes_cache, residual_is_spent=True)
+                if isinstance(need, PagedKvNeed):
+                    ctx.group = cache.group_of[key]
+                    ctx.plane = cache.groups[ctx.group].plane(key)
+                elif isinstance(need, StateNeed):
+                    ctx.state = cache.states[key]
+                x = self.layers[call.layer].forward(x, ctx)
+            x = self.out_norms[j](x)
+        return x
+
     def forward(self, step, cache) -> List[StageOutput]:
-        """Run every stage over its rows; keys, values and state land in `cache`."""
-        outs: List[StageOutput] = []
-        prev = None
-        for j, st in enumerate(self.spec.stages):
-            b = step.stages[j]
-            state = cache.states.get(self.state_keys[j]) if self.state_keys[j] else None
-            x = self.inputs[j].forward(b, prev, self.shared, state)
-            if b.n_rows:
-                for i, call in enumerate(st.calls):
-                    key = self.call_keys[j][i]
-                    need = self.needs.get(key)
-                    # the rows going into a layer are replaced by its result: the layer may overwrite them
-                    ctx = CallContext(batch=b, writes_cache=call.writes_cache, residual_is_spent=True)
-                    if isinstance(need, PagedKvNeed):
-                        ctx.group = cache.group_of[key]
-                        ctx.plane = cache.groups[ctx.group].plane(key)
-                    elif isinstance(need, StateNeed):
-                        ctx.state = cache.states[key]
-                    x = self.layers[call.layer].forward(x, ctx)
-                x = self.out_norms[j](x)
-            prev = x
-            outs.append(StageOutput(x, b))
-        return outs
+        """Run every stage over its rows; keys, values and state land in `cache`.
+
+        A stage that reads the previous one takes each row either from that stage's rows of this step or from
+        the request's state (a row made one step earlier); what a stage keeps for the next step is written after
+        all stages have read. The stages run one after the other on one stream, also in steps of single decoded
+        tokens where they do not depend on one another: as branches of a captured graph they measured slower
+        on MI355X than in sequence (4.3k against 4.5k tokens a second at batch 8).
+        """
+        n = len(self.spec.stages)
+        hidden = [None] * n
+        for j in range(n):
+            hidden[j] = self._run_stage(j, step, cache, hidden[j - 1] if j else None)
+        for j in range(1, n):
+            after = getattr(self.inputs[j], "after_step", None)
+            if after is not None:
+                after(step.stages[j], hidden[j - 1], cache.states.get(self.state_keys[j]) if self.state_keys[j] else None)
+        return [StageOutput(hidden[j], step.stages[j]) for j in range(n)]
 
     def logits(self, hidden, want_index, n):
         """32-bit logits [n, vocab] of the rows `want_index` of `hidden` (reference main_models_new.py:225-226)."""

@@ -59,17 +59,17 @@ class FusePreviousStage:
         self.embed_norm = build_part(spec.params["embed_norm"], tensors, ops)
 
     def forward(self, batch, previous, shared, state):
+        """`previous` may be None when batch.previous_rows is 0: every row then comes from the state."""
         ops, D = self.ops, self.d_model
-        prev_out = previous
-        fused = None
-        if batch.n_rows:
-            fused = ops.empty(batch.n_rows, 2 * D)
-            ops.gather_rows(prev_out, state, batch.source_index, out=fused[:, :D])
-            ops.embedding_rmsnorm(shared["embedding"], batch.tokens, self.embed_norm.gain, self.embed_norm.eps,
-                                  out=fused[:, D:])
-        # after the reads: the previous stage's newest row of each request waits for the next step
-        if batch.keep_count:
-            ops.copy_rows(prev_out, batch.keep_source, state, batch.keep_slot)
-        if fused is None:
+        if not batch.n_rows:
             return ops.empty(0, D)
+        fused = ops.empty(batch.n_rows, 2 * D)
+        ops.gather_rows(previous if previous is not None else state, state, batch.source_index, out=fused[:, :D])
+        ops.embedding_rmsnorm(shared["embedding"], batch.tokens, self.embed_norm.gain, self.embed_norm.eps,
+                              out=fused[:, D:])
         return ops.linear(fused, self.w_proj)
+
+    def after_step(self, batch, previous, state):
+        """Once every stage has read its state: the previous stage's newest row of each request waits for the next step."""
+        if batch.keep_count:
+            self.ops.copy_rows(previous, batch.keep_source, state, batch.keep_slot)

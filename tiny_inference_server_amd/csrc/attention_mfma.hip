@@ -50,7 +50,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
   const int page_size = PS16 ? 16 : page_size_arg;
   const int item = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int lane = threadIdx.x, c16 = lane & 15, g = lane >> 4;
-  const int row0 = items[item].x, n_rows = items[item].y;
+  // no item list: every item is the single row of its own index (a step of decoded tokens), which saves the wave
+  // one of the dependent loads it starts with
+  const int row0 = items ? items[item].x : item, n_rows = items ? items[item].y : 1;
   const int* bt = block_tables + (long)row_seq[row0] * bt_ld;
   const int p_first = positions[row0];
   const int p_last = p_first + n_rows - 1;
@@ -297,36 +299,56 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_kernel(const float* _
                                                                   bf16* __restrict__ out, long out_ld, int n_heads,
                                                                   int n_splits) {
   __shared__ float so[MG][MD][64];
-  __shared__ float sl[MG];
   const long row = blockIdx.x;
   const int head = blockIdx.y;
   const int grp = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long base = (row * n_heads + head) * n_splits;
+  // every wave reads the splits' (maximum, sum) pairs with one split per lane, so that the reads go out together
+  // and not one after the other; the weights stay on the lanes and are handed round by index
   float M = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[base + s].x);
+  for (int s0 = 0; s0 < n_splits; s0 += 64)
+    if (s0 + lane < n_splits) M = fmaxf(M, part_ml[base + s0 + lane].x);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
   float acc[MD];
 #pragma unroll
   for (int j = 0; j < MD; ++j) acc[j] = 0.f;
   float L = 0.f;
-  for (int s = grp; s < n_splits; s += MG) {
-    const float2 ml = part_ml[base + s];
-    if (ml.x == -INFINITY) continue;     // a split that held no key of this row
-    const float w = exp2f(ml.x - M);
-    L += w * ml.y;
+  for (int s0 = 0; s0 < n_splits; s0 += 64) {
+    const int cnt = min(64, n_splits - s0);
+    // the group's partial outputs of this chunk are asked for before the weights are known: one round trip, not two
+    float v[64 / MG][MD];
 #pragma unroll
-    for (int j = 0; j < MD; ++j) {
-      const int d = j * 64 + lane;
-      if (d < HD) acc[j] += w * part_o[(base + s) * HD + d];
+    for (int q = 0; q < 64 / MG; ++q) {
+      const int i = grp + q * MG;
+#pragma unroll
+      for (int j = 0; j < MD; ++j) {
+        const int d = j * 64 + lane;
+        v[q][j] = (i < cnt && d < HD) ? part_o[(base + s0 + i) * HD + d] : 0.f;
+      }
+    }
+    float w = 0.f;
+    if (lane < cnt) {
+      const float2 ml = part_ml[base + s0 + lane];
+      if (ml.x != -INFINITY) {   // else: a split that held no key of this row; its partial output means nothing
+        w = exp2f(ml.x - M);
+        L += w * ml.y;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 64 / MG; ++q) {
+      const float wi = __shfl(w, min(grp + q * MG, 63), 64);
+#pragma unroll
+      for (int j = 0; j < MD; ++j)
+        if (wi != 0.f) acc[j] += wi * v[q][j];
     }
   }
 #pragma unroll
+  for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+#pragma unroll
   for (int j = 0; j < MD; ++j) so[grp][j][lane] = acc[j];
-  if (lane == 0) sl[grp] = L;
   __syncthreads();
   if (grp != 0) return;
-  float Lt = sl[0];
-#pragma unroll
-  for (int gq = 1; gq < MG; ++gq) Lt += sl[gq];
 #pragma unroll
   for (int j = 0; j < MD; ++j) {
     const int d = j * 64 + lane;
@@ -334,14 +356,14 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_kernel(const float* _
     float t = so[0][j][lane];
 #pragma unroll
     for (int gq = 1; gq < MG; ++gq) t += so[gq][j][lane];
-    out[row * out_ld + (long)head * HD + d] = static_cast<__bf16>(t / Lt);
+    out[row * out_ld + (long)head * HD + d] = static_cast<__bf16>(t / L);
   }
 }
 
 TIS_EXPORT int tis_attention_mfma_head_dim() { return HD; }
 
 // items: (first row, rows) pairs; the rows of an item are consecutive positions of one request and
-// rows * group_size <= 16 * nb. part_o / part_ml: workspace for n_splits > 1, [rows][heads][splits][HD] floats and
+// rows * group_size <= 16 * nb. Null: n_items single rows, item i being row i. part_o / part_ml: workspace for n_splits > 1, [rows][heads][splits][HD] floats and
 // [rows][heads][splits] float pairs.
 TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
                                   const int* row_seq, const int* positions, const int* items, int n_items, int nb,

@@ -71,6 +71,30 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
   f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
   float ss = 0.f;
 
+  // What the epilogue wants from memory (the residual; the row's position, rotary factors and cache slot) is asked
+  // for here, by the lanes that will use it, so that its round trips run beside the weights' and not after them.
+  // Result lane (g, c16) of wave 0: columns n_out .. n_out + 3 of row c16.
+  const bool out_lane = wave == 0 && g < GH && c16 < COLS && c16 < M;
+  const int n_out = n0 + g * 4;
+  float res[4] = {0.f, 0.f, 0.f, 0.f};
+  float2 cs[2] = {make_float2(1.f, 0.f), make_float2(1.f, 0.f)};
+  int slot = 0;
+  if (EPI == EPI_RESIDUAL && out_lane) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n_out + i < N) res[i] = static_cast<float>(R_in[(long)c16 * r_ld + n_out + i]);
+  }
+  if (EPI == EPI_ROPE && out_lane && n_out < N) {
+    const int hd = rope.head_dim;
+    const int head = n_out / hd, e0 = n_out % hd;
+    if (head < rope.n_heads + rope.n_kv_heads && rope.table) {
+      const long at = (long)rope.positions[c16] * (hd / 2) + e0 / 2;
+      cs[0] = rope.table[at];
+      cs[1] = rope.table[at + 1];
+    }
+    if (head >= rope.n_heads && rope.write_cache) slot = rope.write_slots[c16];
+  }
+
   // U steps at a time: all their loads are issued before the first product, so that a wave keeps several
   // rows' worth of HBM requests in flight
   for (int s0 = wave; s0 < steps; s0 += U * GS_WAVES) {
@@ -164,10 +188,9 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
           d[2 * j] = rope.interleaved ? 2 * pair : pair;
           d[2 * j + 1] = rope.interleaved ? 2 * pair + 1 : pair + half;
           if (rope.table) {
-            const float2 cs = rope.table[(long)rope.positions[m] * half + pair];
             const float x1 = v[2 * j], x2 = v[2 * j + 1];
-            y[2 * j] = x1 * cs.x - x2 * cs.y;
-            y[2 * j + 1] = x2 * cs.x + x1 * cs.y;
+            y[2 * j] = x1 * cs[j].x - x2 * cs[j].y;
+            y[2 * j + 1] = x2 * cs[j].x + x1 * cs[j].y;
           }
         }
       }
@@ -175,7 +198,6 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) C[(long)m * c_ld + (long)head * hd + d[i]] = from_f<TO>(y[i]);
       } else if (rope.write_cache) {
-        const int slot = rope.write_slots[m];
         const int page = slot / rope.page_size, off = slot % rope.page_size;
         const int kvh = is_v ? head - rope.n_heads - rope.n_kv_heads : head - rope.n_heads;
         bf16* hp = rope.plane + (((long)page * 2 + (is_v ? 1 : 0)) * rope.n_kv_heads + kvh) * rope.page_size * hd;
@@ -198,7 +220,7 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
       for (int i = 0; i < 4; ++i) {
         if (n + i < N) {
           float t = v[i];
-          if (EPI == EPI_RESIDUAL) t += static_cast<float>(R_in[(long)m * r_ld + n + i]);
+          if (EPI == EPI_RESIDUAL) t += res[i];
           C[(long)m * c_ld + n + i] = from_f<TO>(t);
         }
       }

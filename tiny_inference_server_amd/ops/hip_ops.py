@@ -105,13 +105,16 @@ def attention_items(seq_rows, group_size: int):
     """Work items of the matrix-core attention kernel for the rows of one stage.
 
     seq_rows: (first row, first position, rows) per request. Returns (column blocks per item, [(first row, rows)]):
-    an item holds consecutive rows of one request, rows * group_size <= 16 * blocks.
+    an item holds consecutive rows of one request, rows * group_size <= 16 * blocks. When no request has more
+    than one row the list is simply every row in order, which the kernel knows without being given a list.
     """
     single = all(n <= 1 for _, _, n in seq_rows)
     nb = 1 if single else 2
     while group_size > 16 * nb:
         nb *= 2
     per_item = max(1, (16 * nb) // group_size)
+    if single:
+        return nb, [(first, 1) for first, _, n in seq_rows if n]
     items = []
     for first, p0, n in seq_rows:
         for r in range(0, n, per_item):
@@ -472,6 +475,8 @@ class HipOps:
                 items = torch.tensor(host_items, dtype=torch.int32).reshape(-1).to(self.device)
                 plan = (items, len(host_items), nb)
             items, n_items, nb = plan
+            if batch.max_seq_rows <= 1 and n_items == n:
+                items = None        # single rows in order: the kernel needs no list
             lib = self._attn_mfma.get(head_dim)
             if lib is None:
                 lib = self._attn_mfma[head_dim] = library(f"attention_mfma@{head_dim}")

@@ -173,6 +173,28 @@ def test_paged_attention_single_rows(ops_for, dtype, n_heads, n_kv, hd, page_siz
         assert not torch.allclose(got[0].view(n_heads, hd).double(), bad, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("page_size", [16, 32])
+def test_single_rows_walking_a_long_context_without_splits(ops_for, monkeypatch, page_size):
+    """With no key splits one wave walks a request's whole context alone: thousands of keys, hundreds of steps,
+    ending mid-page."""
+    from tiny_inference_server_amd.ops import hip_ops
+    monkeypatch.setattr(hip_ops, "_ATTN_TARGET_WAVES", 1)
+    ops = ops_for(torch.bfloat16)
+    n_heads, n_kv, hd = 4, 2, 64
+    kv_lens = [4097, 9000, 33]
+    plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page_size, torch.bfloat16, seed=25)
+    B = len(kv_lens)
+    q = rnd((B, n_heads * hd), torch.bfloat16, 26)
+    batch = SimpleNamespace(positions=torch.tensor([L - 1 for L in kv_lens], dtype=torch.int32).cuda(),
+                            row_seq=torch.arange(B, dtype=torch.int32).cuda(),
+                            block_tables={"g": tables.cuda()}, max_kv_len=max(kv_lens), extras={},
+                            n_rows=B, max_seq_rows=1, seq_rows=[(i, kv_lens[i] - 1, 1) for i in range(B)])
+    got = ops.paged_attention(q.cuda(), plane.cuda(), batch, "g", n_heads, n_kv, hd).cpu()
+    for i, L in enumerate(kv_lens):
+        want = dense_reference(q[i].view(n_heads, hd), ks[i], vs[i], n_heads // n_kv, L - 1)
+        torch.testing.assert_close(got[i].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_heads,n_kv,hd,page_size", [(4, 2, 64, 16), (3, 1, 32, 8), (12, 3, 128, 16), (2, 2, 48, 16)])
 def test_paged_attention_portions_and_window(ops_for, dtype, n_heads, n_kv, hd, page_size):

@@ -327,9 +327,30 @@ __global__ __launch_bounds__(SM_THREADS) void argmax_kernel(const float* __restr
   const long r = blockIdx.x;
   float mv = -INFINITY;
   int mi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += SM_THREADS) {
-    const float v = logits[r * ld + i];
-    if (v > mv) { mv = v; mi = i; }
+  const float* row = logits + r * ld;
+  if ((((uintptr_t)row) & 15) == 0) {
+    // four values a load, two loads in flight; a thread meets its indices in rising order, so ">" keeps the lowest
+    const int V4 = V & ~3;
+    for (int i = threadIdx.x * 4; i < V4; i += 2 * SM_THREADS * 4) {
+      const int j = i + SM_THREADS * 4;
+      const float4 a = *reinterpret_cast<const float4*>(row + i);
+      const float4 b = j < V4 ? *reinterpret_cast<const float4*>(row + j) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+      const float va[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int at = (e < 4 ? i : j - 4) + e;
+        if (va[e] > mv) { mv = va[e]; mi = at; }
+      }
+    }
+    for (int i = V4 + threadIdx.x; i < V; i += SM_THREADS) {
+      const float v = row[i];
+      if (v > mv || (v == mv && i < mi)) { mv = v; mi = i; }
+    }
+  } else {
+    for (int i = threadIdx.x; i < V; i += SM_THREADS) {
+      const float v = row[i];
+      if (v > mv) { mv = v; mi = i; }
+    }
   }
   block_argmax(mv, mi, sv, si);
   if (threadIdx.x == 0) out_tokens[r] = (mi < 0 || mi >= V) ? 0 : mi;

@@ -1,4 +1,4 @@
-// C[M,N] = f(A[M,K]) . W[N,K]^T for few rows (M <= 16): the matrix product of decode steps, where the job is to
+// C[M,N] = f(A[M,K]) . W[N,K]^T for few rows (M <= 32): the matrix product of decode steps, where the job is to
 // stream W from HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950).
 //
 // One workgroup owns 16 rows of W (16 output columns; 8 in the narrow variant below) over the whole of K; its waves take the 32-wide steps of
@@ -44,62 +44,83 @@ struct RopeArgs {
 // Eight waves of three or four steps measured best on MI355X for K of 1536 to 4096 (5.6 us for a 25 MB matrix,
 // 23 us for the 147 MB output table: 80 % of the HBM peak); four waves where K is too short to feed eight.
 //
+// MB: blocks of 16 rows of X that share every weight tile a wave loads. Two blocks (17 to 32 rows) still beat the
+// library's product plus the separate norm, gate and rotary launches (7.8k against 6.4k tokens a second at batch
+// 20, 9.7k against 9.1k at batch 32); with four blocks the activations, which every workgroup reads in full from
+// L2, outweigh the weights four to one and the library wins (11.2k against 12.8k at batch 64), so four are not built.
+//
 // R: with 16 output columns per workgroup a matrix of 1536 rows gives 96 workgroups, and a compute unit draws
 // only about 24 GB/s, so the 160 idle units cost more than the product. For M <= 16/R rows a workgroup
 // therefore owns only 16/R columns and fills the 16 rows of the matrix operand with R different 32-wide chunks of
 // K for those columns; the activation operand holds the same R chunks side by side. Of the 16x16 result only
 // the R diagonal blocks (chunk r of the weights against chunk r of the activations) mean anything; they are
 // added up with the waves' partial sums. R times as many workgroups, each step covers 32 R of K.
-template <bool NORM, int EPI, typename TO, int GS_WAVES, int U, int R>
+template <int MB, bool NORM, int EPI, typename TO, int GS_WAVES, int U, int R>
 __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
     const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const float* __restrict__ gain, float eps,
     const bf16* __restrict__ R_in, long r_ld, TO* __restrict__ C, long c_ld, int M, int N, int K, RopeArgs rope) {
-  constexpr int COLS = 16 / R;   // output columns of a workgroup, and the most rows of X it takes
+  static_assert(MB == 1 || R == 1, "several row blocks go with full column tiles only");
+  constexpr int COLS = 16 / R;   // output columns of a workgroup, and the most rows of X a block takes
   constexpr int GH = 4 / R;      // lane groups of four result rows per chunk
-  __shared__ float red[GS_WAVES][64][4];
-  __shared__ float red_ss[GS_WAVES][16];
+  __shared__ float red[GS_WAVES][MB][64][4];
+  __shared__ float red_ss[GS_WAVES][MB][16];
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
   const int chunk = c16 / COLS, sub = c16 % COLS;   // the lane's chunk of a step; its weight row and its activation row
   const int n0 = blockIdx.x * COLS;
   const int steps = (K + 32 * R - 1) / (32 * R);
   const bool w_ok = n0 + sub < N;
-  const bool x_ok = sub < M;
   const bf16* wrow = W + (long)(w_ok ? n0 + sub : 0) * K + chunk * 32 + g * 8;
-  const bf16* xrow = X + (long)(x_ok ? sub : 0) * x_ld + chunk * 32 + g * 8;
-
-  f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
-  float ss = 0.f;
+  bool x_ok[MB];
+  const bf16* xrow[MB];
+  f32x4 acc[MB];
+  float ss[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    x_ok[mb] = mb * 16 + sub < M;
+    xrow[mb] = X + (long)(x_ok[mb] ? mb * 16 + sub : 0) * x_ld + chunk * 32 + g * 8;
+    acc[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    ss[mb] = 0.f;
+  }
 
   // What the epilogue wants from memory (the residual; the row's position, rotary factors and cache slot) is asked
   // for here, by the lanes that will use it, so that its round trips run beside the weights' and not after them.
-  // Result lane (g, c16) of wave 0: columns n_out .. n_out + 3 of row c16.
-  const bool out_lane = wave == 0 && g < GH && c16 < COLS && c16 < M;
+  // Result lane (g, c16) of wave 0: columns n_out .. n_out + 3 of the rows mb * 16 + c16.
+  const bool out_lane = wave == 0 && g < GH && c16 < COLS;
   const int n_out = n0 + g * 4;
-  float res[4] = {0.f, 0.f, 0.f, 0.f};
-  float2 cs[2] = {make_float2(1.f, 0.f), make_float2(1.f, 0.f)};
-  int slot = 0;
-  if (EPI == EPI_RESIDUAL && out_lane) {
+  float res[MB][4];
+  float2 cs[MB][2];
+  int slot[MB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (n_out + i < N) res[i] = static_cast<float>(R_in[(long)c16 * r_ld + n_out + i]);
-  }
-  if (EPI == EPI_ROPE && out_lane && n_out < N) {
-    const int hd = rope.head_dim;
-    const int head = n_out / hd, e0 = n_out % hd;
-    if (head < rope.n_heads + rope.n_kv_heads && rope.table) {
-      const long at = (long)rope.positions[c16] * (hd / 2) + e0 / 2;
-      cs[0] = rope.table[at];
-      cs[1] = rope.table[at + 1];
+  for (int mb = 0; mb < MB; ++mb) {
+    const int m = mb * 16 + c16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) res[mb][i] = 0.f;
+    cs[mb][0] = cs[mb][1] = make_float2(1.f, 0.f);
+    slot[mb] = 0;
+    if (!out_lane || m >= M) continue;
+    if (EPI == EPI_RESIDUAL) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n_out + i < N) res[mb][i] = static_cast<float>(R_in[(long)m * r_ld + n_out + i]);
     }
-    if (head >= rope.n_heads && rope.write_cache) slot = rope.write_slots[c16];
+    if (EPI == EPI_ROPE && n_out < N) {
+      const int hd = rope.head_dim;
+      const int head = n_out / hd, e0 = n_out % hd;
+      if (head < rope.n_heads + rope.n_kv_heads && rope.table) {
+        const long at = (long)rope.positions[m] * (hd / 2) + e0 / 2;
+        cs[mb][0] = rope.table[at];
+        cs[mb][1] = rope.table[at + 1];
+      }
+      if (head >= rope.n_heads && rope.write_cache) slot[mb] = rope.write_slots[m];
+    }
   }
 
   // U steps at a time: all their loads are issued before the first product, so that a wave keeps several
   // rows' worth of HBM requests in flight
   for (int s0 = wave; s0 < steps; s0 += U * GS_WAVES) {
     bf16x8 a[U];
-    bf16x8 b[U];
+    bf16x8 b[U][MB];
     float gv[U][8];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -107,9 +128,12 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
       const int k = s * (32 * R) + chunk * 32 + g * 8;
       const bool k_ok = s < steps && k < K;   // K is a multiple of 8, so a lane's 8 values are all inside or all outside
       a[u] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-      b[u] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
       if (w_ok && k_ok) a[u] = *reinterpret_cast<const bf16x8*>(wrow + (long)s * (32 * R));
-      if (x_ok && k_ok) b[u] = *reinterpret_cast<const bf16x8*>(xrow + (long)s * (32 * R));
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        b[u][mb] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+        if (x_ok[mb] && k_ok) b[u][mb] = *reinterpret_cast<const bf16x8*>(xrow[mb] + (long)s * (32 * R));
+      }
       if (NORM) {
         const float4 g0 = k_ok ? *reinterpret_cast<const float4*>(gain + k) : make_float4(0.f, 0.f, 0.f, 0.f);
         const float4 g1 = k_ok ? *reinterpret_cast<const float4*>(gain + k + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -119,60 +143,69 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      bf16x8 bv = b[u];
-      if (NORM) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float xf = static_cast<float>(bv[e]);
-          ss += xf * xf;
-          bv[e] = static_cast<__bf16>(xf * gv[u][e]);
+      for (int mb = 0; mb < MB; ++mb) {
+        bf16x8 bv = b[u][mb];
+        if (NORM) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float xf = static_cast<float>(bv[e]);
+            ss[mb] += xf * xf;
+            bv[e] = static_cast<__bf16>(xf * gv[u][e]);
+          }
         }
+        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc[mb], 0, 0, 0);
       }
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc, 0, 0, 0);
     }
   }
 
   // add the partial sums of the waves and of the chunks in a fixed order
 #pragma unroll
-  for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
-  if (NORM) {
-    float t = ss;
-    t += __shfl_xor(t, 16, 64);
-    t += __shfl_xor(t, 32, 64);
-    if (g == 0) red_ss[wave][c16] = t;
+  for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][mb][lane][i] = acc[mb][i];
+    if (NORM) {
+      float t = ss[mb];
+      t += __shfl_xor(t, 16, 64);
+      t += __shfl_xor(t, 32, 64);
+      if (g == 0) red_ss[wave][mb][c16] = t;
+    }
   }
   __syncthreads();
   if (wave != 0) return;
-  // result lane (gh, m): columns n0 + 4 gh + i of row m; chunk r's share sits with lane (r GH + gh, r COLS + m)
-  const int gh = lane >> 4, m = lane & 15;
-  if (gh >= GH || m >= COLS || m >= M) return;
-  float v[4];
+  // result lane (gh, c): columns n0 + 4 gh + i of the rows mb * 16 + c; chunk r's share sits with lane (r GH + gh, r COLS + c)
+  const int gh = lane >> 4, c = lane & 15;
+  if (gh >= GH || c >= COLS) return;
+  const int n = n0 + gh * 4;   // the lane's four consecutive output columns
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    float t = 0.f;
+  for (int mb = 0; mb < MB; ++mb) {
+    const int m = mb * 16 + c;
+    if (m >= M) continue;
+    float v[4];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int src = (r * GH + gh) * 16 + r * COLS + m;
+    for (int i = 0; i < 4; ++i) {
+      float t = 0.f;
 #pragma unroll
-      for (int w = 0; w < GS_WAVES; ++w) t += red[w][src][i];
+      for (int r = 0; r < R; ++r) {
+        const int src = (r * GH + gh) * 16 + r * COLS + c;
+#pragma unroll
+        for (int w = 0; w < GS_WAVES; ++w) t += red[w][mb][src][i];
+      }
+      v[i] = t;
     }
-    v[i] = t;
-  }
-  if (NORM) {
-    float t = 0.f;
+    if (NORM) {
+      float t = 0.f;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
+      for (int r = 0; r < R; ++r) {
 #pragma unroll
-      for (int w = 0; w < GS_WAVES; ++w) t += red_ss[w][r * COLS + m];
+        for (int w = 0; w < GS_WAVES; ++w) t += red_ss[w][mb][r * COLS + c];
+      }
+      const float mul = sqrtf((float)K) / (sqrtf(t) + eps);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= mul;
     }
-    const float mul = sqrtf((float)K) / (sqrtf(t) + eps);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] *= mul;
-  }
-  {
-    const int n = n0 + gh * 4;   // the lane's four consecutive output columns
     if (EPI == EPI_ROPE) {
-      if (n >= N) return;          // N is a multiple of head_dim, head_dim of 4: the lane's columns are all in or out
+      if (n >= N) continue;          // N is a multiple of head_dim, head_dim of 4: the lane's columns are all in or out
       const int hd = rope.head_dim, half = hd / 2;
       const int head = n / hd, e0 = n % hd;      // e0 is a multiple of 4: two whole pairs
       const bool is_q = head < rope.n_heads, is_v = head >= rope.n_heads + rope.n_kv_heads;
@@ -189,8 +222,8 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
           d[2 * j + 1] = rope.interleaved ? 2 * pair + 1 : pair + half;
           if (rope.table) {
             const float x1 = v[2 * j], x2 = v[2 * j + 1];
-            y[2 * j] = x1 * cs[j].x - x2 * cs[j].y;
-            y[2 * j + 1] = x2 * cs[j].x + x1 * cs[j].y;
+            y[2 * j] = x1 * cs[mb][j].x - x2 * cs[mb][j].y;
+            y[2 * j + 1] = x2 * cs[mb][j].x + x1 * cs[mb][j].y;
           }
         }
       }
@@ -198,7 +231,7 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) C[(long)m * c_ld + (long)head * hd + d[i]] = from_f<TO>(y[i]);
       } else if (rope.write_cache) {
-        const int page = slot / rope.page_size, off = slot % rope.page_size;
+        const int page = slot[mb] / rope.page_size, off = slot[mb] % rope.page_size;
         const int kvh = is_v ? head - rope.n_heads - rope.n_kv_heads : head - rope.n_heads;
         bf16* hp = rope.plane + (((long)page * 2 + (is_v ? 1 : 0)) * rope.n_kv_heads + kvh) * rope.page_size * hd;
 #pragma unroll
@@ -220,7 +253,7 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
       for (int i = 0; i < 4; ++i) {
         if (n + i < N) {
           float t = v[i];
-          if (EPI == EPI_RESIDUAL) t += res[i];
+          if (EPI == EPI_RESIDUAL) t += res[mb][i];
           C[(long)m * c_ld + n + i] = from_f<TO>(t);
         }
       }
@@ -236,6 +269,7 @@ TIS_EXPORT void tis_gemm_skinny_force_config(int waves, int u, int r) {
   g_force_r = r;
 }
 
+
 template <bool NORM, int EPI, typename TO>
 static int launch(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
                   void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope = RopeArgs()) {
@@ -245,7 +279,8 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
   int r = (M <= 8 && (N + 15) / 16 <= 128) ? 2 : 1;
   if (g_force_r) r = g_force_r;
   if (r != 1 && r != 2) return tis_fail("gemm_skinny: %d chunks a step; 1 or 2 are built", r);
-  if (M > 16 / r) return tis_fail("gemm_skinny: %d rows do not fit %d columns a workgroup", M, 16 / r);
+  if (r == 2 && M > 8) return tis_fail("gemm_skinny: %d rows do not fit 8 columns a workgroup", M);
+  const int mb = M <= 16 ? 1 : 2;
   const int steps = (K + 32 * r - 1) / (32 * r);
   int waves, u;
   if (steps >= 24) {
@@ -257,26 +292,26 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
     u = (steps % 3 == 0 && steps % 4 != 0) || steps == 12 ? 3 : 4;
   }
   if (g_force_waves) { waves = g_force_waves; u = g_force_u; }
+  if (mb > 1 && waves != 8) { waves = 8; u = 4; }   // several row blocks are built for eight waves only
   const int cols = 16 / r;
   const int n_wg = (N + cols - 1) / cols;
-#define CFG(WV, UV, RV)                                                                                          \
-  if (waves == WV && u == UV && r == RV) {                                                                       \
-    gemm_skinny_kernel<NORM, EPI, TO, WV, UV, RV><<<n_wg, WV * 64, 0, stream>>>(                                 \
+#define CFG(MBV, WV, UV, RV)                                                                                     \
+  if (mb == MBV && waves == WV && u == UV && r == RV) {                                                          \
+    gemm_skinny_kernel<MBV, NORM, EPI, TO, WV, UV, RV><<<n_wg, WV * 64, 0, stream>>>(                            \
         (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);     \
     return 0;                                                                                                    \
   }
-#define CFGS(RV) CFG(4, 3, RV) CFG(4, 4, RV) CFG(8, 3, RV) CFG(8, 4, RV)
+#define CFGS(RV) CFG(1, 4, 3, RV) CFG(1, 4, 4, RV) CFG(1, 8, 3, RV) CFG(1, 8, 4, RV)
   CFGS(1) CFGS(2)
+  CFG(2, 8, 3, 1) CFG(2, 8, 4, 1)
 #undef CFGS
 #undef CFG
-  return tis_fail("gemm_skinny: no kernel for %d waves of %d steps and %d chunks", waves, u, r);
+  return tis_fail("gemm_skinny: no kernel for %d row blocks, %d waves of %d steps and %d chunks", mb, waves, u, r);
 }
 
 template <bool NORM, int EPI, typename TO>
 static int launch_mb(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
                      void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope = RopeArgs()) {
-  // 16 rows at most: with more rows the library's product is faster than this kernel even after paying for
-  // the separate norm, gating and rotary launches
   if (launch<NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope)) return -1;
   return tis_launch_status("gemm_skinny");
 }
@@ -286,7 +321,7 @@ TIS_EXPORT int tis_gemm_skinny(const void* X, long x_ld, const void* W, const fl
                                long r_ld, void* C, long c_ld, int M, int N, int K, int epilogue, int out_dtype,
                                hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
-  if (M < 0 || M > 16) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..16", M);
+  if (M < 0 || M > 32) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..32", M);
   if (N < 1 || K < 8 || K % 8) return tis_fail("gemm_skinny: N=%d K=%d; K must be a multiple of 8", N, K);
   if (x_ld % 8 || ((uintptr_t)X % 16) || ((uintptr_t)W % 16))
     return tis_fail("gemm_skinny: activations and weights must be 16-byte aligned with row strides in steps of 8");
@@ -312,7 +347,7 @@ TIS_EXPORT int tis_gemm_skinny_qkv_rope(const void* X, long x_ld, const void* W,
                                         const float* table, void* plane, int n_heads, int n_kv_heads, int head_dim,
                                         int page_size, int interleaved, int write_cache, hipStream_t stream) {
   if (M == 0) return 0;
-  if (M < 0 || M > 16) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..16", M);
+  if (M < 0 || M > 32) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..32", M);
   if (K < 8 || K % 8) return tis_fail("gemm_skinny: K=%d must be a multiple of 8", K);
   if (n_heads < 1 || n_kv_heads < 1 || head_dim < 4 || head_dim % 4 || page_size < 1)
     return tis_fail("gemm_skinny: heads=%d kv_heads=%d head_dim=%d (a multiple of 4) page=%d", n_heads, n_kv_heads,

@@ -95,7 +95,7 @@ def library(name: str) -> _Lib:
 
 
 # wavefronts the attention launch aims for, so that short batches still spread over the chip
-_SKINNY_MAX_ROWS = 16
+_SKINNY_MAX_ROWS = 32
 _ATTN_TARGET_WAVES = 512
 _ATTN_MIN_SPLIT_KEYS = 128      # a split shorter than this costs more in merging than it gains in spreading
 _ATTN_WORKSPACE_FLOATS = 16 << 20
@@ -328,7 +328,7 @@ class HipOps:
         return self._linear_bf16(x, w, residual, out_dtype, reuse_residual)
 
     def _skinny_ok(self, x, M, K):
-        # up to 16 rows the fused few-row kernel wins (it saves the norm, gating and rotary launches and streams the
+        # up to 32 rows the fused few-row kernel wins (it saves the norm, gating and rotary launches and streams the
         # weights as fast as the library does); beyond, the library's product is enough faster to pay for them
         return (self.dtype == torch.bfloat16 and 0 < M <= _SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0
                 and x.data_ptr() % 16 == 0)

@@ -223,6 +223,34 @@ def test_paged_attention_portions_and_window(ops_for, dtype, n_heads, n_kv, hd, 
             torch.testing.assert_close(got[r].view(n_heads, hd).double(), want, **t)
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,page_size", [(12, 3, 128, 16), (32, 8, 32, 16), (4, 2, 64, 32)])
+def test_mixed_rows_with_key_splits_chosen_item_by_item(ops_for, n_heads, n_kv, hd, page_size):
+    """A small batch of prompt rows and single rows far into long requests: the keys are cut into splits, every item
+    takes as many as its own length deserves (some one, some many), and the merge reads each row's count. With 32
+    heads the rows times heads pass the size at which the merge goes row by row."""
+    ops = ops_for(torch.bfloat16)
+    group = n_heads // n_kv
+    kv_lens = [1500, 1340, 40, 9, 700]
+    plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page_size, torch.bfloat16, seed=33)
+    # request 0: its last row; request 1: rows 1040..1339 (a portion deep into a prompt); request 2: a whole short
+    # prompt; request 3: its last row, nine keys in all; request 4: its last row
+    segs = [(0, 1499, 1), (1, 1040, 300), (2, 0, 40), (3, 8, 1), (4, 699, 1)]
+    positions, row_seq, seq_rows = [], [], []
+    for s_, p0, n in segs:
+        seq_rows.append((len(positions), p0, n))
+        positions += list(range(p0, p0 + n)); row_seq += [s_] * n
+    R = len(positions)
+    q = rnd((R, n_heads * hd), torch.bfloat16, 34)
+    batch = SimpleNamespace(positions=torch.tensor(positions, dtype=torch.int32).cuda(),
+                            row_seq=torch.tensor(row_seq, dtype=torch.int32).cuda(),
+                            block_tables={"g": tables.cuda()}, max_kv_len=max(kv_lens), extras={},
+                            n_rows=R, max_seq_rows=300, seq_rows=seq_rows)
+    got = ops.paged_attention(q.cuda(), plane.cuda(), batch, "g", n_heads, n_kv, hd).cpu()
+    for r in list(range(0, R, 11)) + [0, 1, 300, 301, 340, 341, R - 1]:
+        want = dense_reference(q[r].view(n_heads, hd), ks[row_seq[r]], vs[row_seq[r]], group, positions[r])
+        torch.testing.assert_close(got[r].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_one_far_key_among_hundreds(ops_for, dtype):
     """One key far back is made to dominate: a kernel that skips a page or a split would miss it."""

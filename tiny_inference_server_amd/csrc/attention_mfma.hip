@@ -46,7 +46,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     const bf16* __restrict__ q, long q_ld, const bf16* __restrict__ plane, const int* __restrict__ block_tables,
     int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ items,
     bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
-    int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits) {
+    int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits, int min_steps,
+    int* __restrict__ row_splits) {
   const int page_size = PS16 ? 16 : page_size_arg;
   const int item = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int lane = threadIdx.x, c16 = lane & 15, g = lane >> 4;
@@ -89,7 +90,15 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
   const int k_hi = p_last + 1;
   const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;   // the largest window start
   const int n_steps = (k_hi - k_lo + 31) / 32;
-  const int per_split = (n_steps + n_splits - 1) / n_splits;
+  // The grid offers every item n_splits waves a kv head. With min_steps an item takes only as many of them as
+  // leaves each at least that many steps, so that short items are not cut into crumbs while long ones (the last
+  // rows of a prompt, whose chain of steps would otherwise set the kernel's time) are; the rest return at once.
+  // row_splits tells the merge how many partial results each row has (one: the output is already final).
+  int item_splits = n_splits;
+  if (min_steps > 0) item_splits = max(1, min(n_splits, n_steps / min_steps));
+  if (split >= item_splits) return;
+  if (row_splits && kvh == 0 && split == 0 && lane < n_rows) row_splits[row0 + lane] = item_splits;
+  const int per_split = (n_steps + item_splits - 1) / item_splits;
   const int s_begin = split * per_split;
   const int s_end = min(n_steps, s_begin + per_split);
 
@@ -168,6 +177,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     // mask, running maximum and sum per column, P in bfloat16 as the B operand of the second product.
     // A step whose 32 keys lie inside every column's range needs no mask at all (most steps of a long row).
     const bool full = T.ok[0] && T.ok[1] && kb + 31 <= p_first && kb >= lo_last;
+    if (!full) {
+      // one branch a step around all the masking, not one around each score
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = kb + t * 16 + g * 4 + i;
+            const bool ok = T.ok[t] && key <= col_pos[nb] && key >= col_lo[nb];
+            st[t][nb][i] = ok ? st[t][nb][i] : -INFINITY;
+          }
+    }
     bf16x8 pb[NB];
     float alpha[NB];
     bool grew = false;
@@ -179,12 +201,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          float v = st[t][nb][i];         // unscaled: the scale (positive) goes into the exponent's multiply-add
-          if (!full) {
-            const int key = kb + t * 16 + g * 4 + i;
-            const bool ok = T.ok[t] && key <= col_pos[nb] && key >= col_lo[nb];
-            v = ok ? v : -INFINITY;
-          }
+          const float v = st[t][nb][i];   // unscaled: the scale (positive) goes into the exponent's multiply-add
           sv[t * 4 + i] = v;
           tmax = fmaxf(tmax, v);
         }
@@ -230,8 +247,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
   };
 
   if (NB >= 2) {
-    // Wide items (rows of prompt portions) are bound by arithmetic, not by memory: they keep one step's tiles only,
-    // which leaves registers for a second wave per SIMD to fill the gaps, and prefetch just the page ids.
+    // Wide items (rows of prompt portions) are bound by instruction issue, not by memory: they keep one step's
+    // tiles only, which leaves registers for a second wave per SIMD to fill the gaps, and prefetch just the page
+    // ids. (A second set of tiles to load ahead into would live in accumulator registers and cost some 180 copy
+    // instructions a step: measured slower even where a wave has its SIMD to itself.)
     if (s_begin < s_end) {
       Tiles ta;
       int pa[2], pn[2];
@@ -268,7 +287,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (!col_ok[nb]) continue;
-    if (n_splits == 1) {
+    if (item_splits == 1) {
       const float inv = 1.f / lt;
       bf16* dst = out + (long)col_row[nb] * out_ld + (long)col_head[nb] * HD + g * 4;
 #pragma unroll
@@ -297,12 +316,14 @@ static constexpr int MD = (HD + 63) / 64;  // outputs per lane
 __global__ __launch_bounds__(MG * 64) void attention_merge_kernel(const float* __restrict__ part_o,
                                                                   const float2* __restrict__ part_ml,
                                                                   bf16* __restrict__ out, long out_ld, int n_heads,
-                                                                  int n_splits) {
+                                                                  int max_splits, const int* __restrict__ row_splits) {
   __shared__ float so[MG][MD][64];
   const long row = blockIdx.x;
   const int head = blockIdx.y;
   const int grp = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const long base = (row * n_heads + head) * n_splits;
+  const int n_splits = row_splits ? row_splits[row] : max_splits;   // partial results of this row
+  if (n_splits <= 1) return;                                        // its output is final already
+  const long base = (row * n_heads + head) * max_splits;
   // every wave reads the splits' (maximum, sum) pairs with one split per lane, so that the reads go out together
   // and not one after the other; the weights stay on the lanes and are handed round by index
   float M = -INFINITY;
@@ -360,16 +381,68 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_kernel(const float* _
   }
 }
 
+// The same merge for many rows (prompt portions): one workgroup a row, its four waves take the heads in turn, and a
+// row that was not split costs one load. With a workgroup per (row, head) the thousands of rows of a prompt would
+// mean tens of thousands of workgroups that each live for three round trips to memory.
+__global__ __launch_bounds__(MG * 64) void attention_merge_rows_kernel(const float* __restrict__ part_o,
+                                                                       const float2* __restrict__ part_ml,
+                                                                       bf16* __restrict__ out, long out_ld,
+                                                                       int n_heads, int max_splits,
+                                                                       const int* __restrict__ row_splits) {
+  const long row = blockIdx.x;
+  const int n_splits = row_splits ? row_splits[row] : max_splits;
+  if (n_splits <= 1) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int head = wave; head < n_heads; head += MG) {
+    const long base = (row * n_heads + head) * max_splits;
+    float acc[MD];
+#pragma unroll
+    for (int j = 0; j < MD; ++j) acc[j] = 0.f;
+    float M = -INFINITY, L = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += 64)
+      if (s0 + lane < n_splits) M = fmaxf(M, part_ml[base + s0 + lane].x);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+    for (int s0 = 0; s0 < n_splits; s0 += 64) {
+      float w = 0.f;
+      if (s0 + lane < n_splits) {
+        const float2 ml = part_ml[base + s0 + lane];
+        if (ml.x != -INFINITY) {
+          w = exp2f(ml.x - M);
+          L += w * ml.y;
+        }
+      }
+      const int cnt = min(64, n_splits - s0);
+      for (int i = 0; i < cnt; ++i) {
+        const float wi = __shfl(w, i, 64);
+#pragma unroll
+        for (int j = 0; j < MD; ++j) {
+          const int d = j * 64 + lane;
+          if (d < HD && wi != 0.f) acc[j] += wi * part_o[(base + s0 + i) * HD + d];
+        }
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+#pragma unroll
+    for (int j = 0; j < MD; ++j) {
+      const int d = j * 64 + lane;
+      if (d < HD) out[row * out_ld + (long)head * HD + d] = static_cast<__bf16>(acc[j] / L);
+    }
+  }
+}
+
 TIS_EXPORT int tis_attention_mfma_head_dim() { return HD; }
 
 // items: (first row, rows) pairs; the rows of an item are consecutive positions of one request and
-// rows * group_size <= 16 * nb. Null: n_items single rows, item i being row i. part_o / part_ml: workspace for n_splits > 1, [rows][heads][splits][HD] floats and
-// [rows][heads][splits] float pairs.
+// rows * group_size <= 16 * nb. Null: n_items single rows, item i being row i. part_o / part_ml: workspace for
+// n_splits > 1, [rows][heads][splits][HD] floats and [rows][heads][splits] float pairs. min_steps > 0: an item
+// uses min(n_splits, its steps of 32 keys / min_steps) splits, and row_splits [rows] receives each row's count.
 TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
                                   const int* row_seq, const int* positions, const int* items, int n_items, int nb,
                                   void* out, long out_ld, float* part_o, float* part_ml, int rows, int n_heads,
                                   int n_kv_heads, int head_dim, int page_size, int window, float scale, int n_splits,
-                                  hipStream_t stream) {
+                                  int min_steps, int* row_splits, hipStream_t stream) {
   if (n_items == 0 || rows == 0) return 0;
   if (head_dim != HD) return tis_fail("attention_mfma: built for head size %d, called with %d", HD, head_dim);
   if (n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads)
@@ -380,6 +453,9 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
   if (page_size < 16 || page_size % 16) return tis_fail("attention_mfma: page size %d is no multiple of 16", page_size);
   if (n_splits < 1 || n_splits > 65535 || n_kv_heads > 65535) return tis_fail("attention_mfma: bad grid %d x %d", n_kv_heads, n_splits);
   if (n_splits > 1 && (!part_o || !part_ml)) return tis_fail("attention_mfma: %d splits need a workspace", n_splits);
+  if (min_steps < 0 || (min_steps > 0 && n_splits > 1 && !row_splits))
+    return tis_fail("attention_mfma: splits chosen item by item (min_steps=%d) need the per-row count array", min_steps);
+  if (min_steps == 0 || n_splits == 1) row_splits = nullptr;
   if ((q_ld % 8) || (out_ld % 4) || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)plane % 16))
     return tis_fail("attention_mfma: q, out and the cache plane must be 16-byte aligned with row strides in steps of 8");
   dim3 grid(n_items, n_kv_heads, n_splits);
@@ -388,7 +464,7 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
   attention_mfma_kernel<NBV, PSV><<<grid, 64, 0, stream>>>(                                                      \
       (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)items,     \
       (bf16*)out, out_ld, part_o, (float2*)part_ml, group, n_kv_heads, n_heads, page_size, window, scale_log2,   \
-      n_splits)
+      n_splits, min_steps, row_splits)
   if (page_size == 16) {
     if (nb == 1) LAUNCH(1, true);
     else if (nb == 2) LAUNCH(2, true);
@@ -402,9 +478,14 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
   int rc = tis_launch_status("attention_mfma");
   if (rc) return rc;
   if (n_splits > 1) {
-    dim3 mgrid(rows, n_heads);
-    attention_merge_kernel<<<mgrid, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld, n_heads,
-                                                          n_splits);
+    if ((long)rows * n_heads > 8192) {
+      attention_merge_rows_kernel<<<rows, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld,
+                                                                n_heads, n_splits, row_splits);
+    } else {
+      dim3 mgrid(rows, n_heads);
+      attention_merge_kernel<<<mgrid, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld,
+                                                            n_heads, n_splits, row_splits);
+    }
     rc = tis_launch_status("attention_merge");
   }
   return rc;

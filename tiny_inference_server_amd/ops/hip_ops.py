@@ -79,7 +79,8 @@ _SIGNATURES["gemm_skinny"] = ("tis_gemm_skinny", {
     "tis_gemm_skinny_qkv_rope": [_P, _L, _P, _P, _F, _P, _L, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
 })
 _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
-    "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I,
+                           _P, _P],
 })
 
 _libs = {}
@@ -97,6 +98,9 @@ def library(name: str) -> _Lib:
 # wavefronts the attention launch aims for, so that short batches still spread over the chip
 _SKINNY_MAX_ROWS = 32
 _ATTN_TARGET_WAVES = 512
+_ATTN_PROMPT_TARGET_WAVES = 2048  # what the grid offers where rows of prompts are in the batch ...
+_ATTN_PROMPT_SPLIT_MAX_ROWS = 512 # ... and the batch is small; a long portion fills the chip by its rows alone
+_ATTN_PROMPT_MIN_STEPS = 8         # steps of 32 keys below which a prompt item's split is not worth its merge
 _ATTN_MIN_SPLIT_KEYS = 128      # a split shorter than this costs more in merging than it gains in spreading
 _ATTN_WORKSPACE_FLOATS = 16 << 20
 
@@ -110,6 +114,10 @@ def attention_items(seq_rows, group_size: int):
     """
     single = all(n <= 1 for _, _, n in seq_rows)
     nb = 1 if single else 2
+    # 64-column items halve what a prompt reads of its keys and values; they pay (some 10 % at 8,192 rows) once
+    # there are enough of them to fill the chip, and cost where a few long chains of steps set the time
+    if not single and group_size <= 64 and sum(-(-n // max(1, 64 // group_size)) for _, _, n in seq_rows) >= 384:
+        nb = 4
     while group_size > 16 * nb:
         nb *= 2
     per_item = max(1, (16 * nb) // group_size)
@@ -480,12 +488,18 @@ class HipOps:
             lib = self._attn_mfma.get(head_dim)
             if lib is None:
                 lib = self._attn_mfma[head_dim] = library(f"attention_mfma@{head_dim}")
-            n_splits = max(1, min(-(-_ATTN_TARGET_WAVES // (n_items * n_kv_heads)),
-                                  batch.max_kv_len // _ATTN_MIN_SPLIT_KEYS))
+            single = items is None
+            # decoded tokens: every request's keys are cut into the same number of splits, enough to spread a short
+            # batch over the chip. Prompt rows: the grid offers more splits than the chip needs and every item takes
+            # as many as its own length deserves (the kernel decides, from _ATTN_PROMPT_MIN_STEPS), because the last
+            # rows of a long prompt would otherwise run on alone long after the first have finished.
+            target = _ATTN_PROMPT_TARGET_WAVES if (not single and n <= _ATTN_PROMPT_SPLIT_MAX_ROWS) else _ATTN_TARGET_WAVES
+            n_splits = max(1, min(-(-target // (n_items * n_kv_heads)), batch.max_kv_len // _ATTN_MIN_SPLIT_KEYS))
+            min_steps = 0 if single else _ATTN_PROMPT_MIN_STEPS
             # partial results of split key ranges live in one workspace of fixed size, allocated once and never
             # moved (captured graphs hold its address); fewer splits where it would not suffice
-            n_splits = max(1, min(n_splits, _ATTN_WORKSPACE_FLOATS // (n * n_heads * (head_dim + 2))))
-            part_o = part_ml = None
+            n_splits = max(1, min(n_splits, (_ATTN_WORKSPACE_FLOATS - n) // (n * n_heads * (head_dim + 2))))
+            part_o = part_ml = row_splits = None
             if n_splits > 1:
                 if self._workspace is None:
                     if torch.cuda.is_current_stream_capturing():
@@ -493,10 +507,13 @@ class HipOps:
                     self._workspace = torch.empty(_ATTN_WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
                 part_o = self._workspace
                 part_ml = self._workspace[n * n_heads * n_splits * head_dim:]
+                if min_steps:
+                    row_splits = self._workspace[n * n_heads * n_splits * (head_dim + 2):]
             lib.tis_attention_mfma(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0),
                                    _ptr(batch.row_seq), _ptr(batch.positions), _ptr(items), n_items, nb, _ptr(out),
                                    out.stride(0), _ptr(part_o), _ptr(part_ml), n, n_heads, n_kv_heads, head_dim,
-                                   page_size, int(window), float(scale), n_splits, self._stream())
+                                   page_size, int(window), float(scale), n_splits, min_steps, _ptr(row_splits),
+                                   self._stream())
             return out
         self.attn_generic.tis_attention_generic(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),

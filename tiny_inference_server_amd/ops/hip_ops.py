@@ -494,7 +494,9 @@ class HipOps:
             # as many as its own length deserves (the kernel decides, from _ATTN_PROMPT_MIN_STEPS), because the last
             # rows of a long prompt would otherwise run on alone long after the first have finished.
             target = _ATTN_PROMPT_TARGET_WAVES if (not single and n <= _ATTN_PROMPT_SPLIT_MAX_ROWS) else _ATTN_TARGET_WAVES
-            n_splits = max(1, min(-(-target // (n_items * n_kv_heads)), batch.max_kv_len // _ATTN_MIN_SPLIT_KEYS))
+            # a lone request or two: shorter splits still pay, because so few waves would leave most of the chip idle
+            min_keys = _ATTN_MIN_SPLIT_KEYS // 2 if n_items * n_kv_heads <= 8 else _ATTN_MIN_SPLIT_KEYS
+            n_splits = max(1, min(-(-target // (n_items * n_kv_heads)), batch.max_kv_len // min_keys))
             min_steps = 0 if single else _ATTN_PROMPT_MIN_STEPS
             # partial results of split key ranges live in one workspace of fixed size, allocated once and never
             # moved (captured graphs hold its address); fewer splits where it would not suffice

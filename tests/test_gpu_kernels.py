@@ -394,7 +394,7 @@ def test_skinny_product_with_fused_norm_residual_and_gate(ops_for, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M", [1, 5, 16, 64, 200])
+@pytest.mark.parametrize("M", [1, 5, 16, 27, 33, 64, 65, 200])
 @pytest.mark.parametrize("n_heads,n_kv,hd,page_size,interleaved", [(8, 2, 8, 16, False), (3, 1, 32, 8, False),
                                                                     (12, 3, 128, 16, False), (4, 2, 48, 16, True)])
 def test_projection_with_rotary_and_cache_write(ops_for, dtype, M, n_heads, n_kv, hd, page_size, interleaved):

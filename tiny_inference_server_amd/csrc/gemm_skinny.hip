@@ -47,7 +47,9 @@ struct RopeArgs {
 // MB: blocks of 16 rows of X that share every weight tile a wave loads. Two blocks (17 to 32 rows) still beat the
 // library's product plus the separate norm, gate and rotary launches (7.8k against 6.4k tokens a second at batch
 // 20, 9.7k against 9.1k at batch 32); with four blocks the activations, which every workgroup reads in full from
-// L2, outweigh the weights four to one and the library wins (11.2k against 12.8k at batch 64), so four are not built.
+// L2, outweigh the weights four to one and the library wins (11.2k against 12.8k at batch 64), except for the
+// q/k/v projection, where this kernel stands for three launches (norm, product, rotary with cache write: 12.9k
+// against 12.7k at batch 64, 11.5k against 11.1k at batch 48); four blocks are built for that one only.
 //
 // R: with 16 output columns per workgroup a matrix of 1536 rows gives 96 workgroups, and a compute unit draws
 // only about 24 GB/s, so the 160 idle units cost more than the product. For M <= 16/R rows a workgroup
@@ -280,7 +282,7 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
   if (g_force_r) r = g_force_r;
   if (r != 1 && r != 2) return tis_fail("gemm_skinny: %d chunks a step; 1 or 2 are built", r);
   if (r == 2 && M > 8) return tis_fail("gemm_skinny: %d rows do not fit 8 columns a workgroup", M);
-  const int mb = M <= 16 ? 1 : 2;
+  const int mb = M <= 16 ? 1 : M <= 32 ? 2 : 4;
   const int steps = (K + 32 * r - 1) / (32 * r);
   int waves, u;
   if (steps >= 24) {
@@ -304,6 +306,7 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
 #define CFGS(RV) CFG(1, 4, 3, RV) CFG(1, 4, 4, RV) CFG(1, 8, 3, RV) CFG(1, 8, 4, RV)
   CFGS(1) CFGS(2)
   CFG(2, 8, 3, 1) CFG(2, 8, 4, 1)
+  if constexpr (EPI == EPI_ROPE) { CFG(4, 8, 3, 1) CFG(4, 8, 4, 1) }   // four blocks: built for the q/k/v projection only
 #undef CFGS
 #undef CFG
   return tis_fail("gemm_skinny: no kernel for %d row blocks, %d waves of %d steps and %d chunks", mb, waves, u, r);
@@ -347,7 +350,7 @@ TIS_EXPORT int tis_gemm_skinny_qkv_rope(const void* X, long x_ld, const void* W,
                                         const float* table, void* plane, int n_heads, int n_kv_heads, int head_dim,
                                         int page_size, int interleaved, int write_cache, hipStream_t stream) {
   if (M == 0) return 0;
-  if (M < 0 || M > 32) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..32", M);
+  if (M < 0 || M > 64) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..64", M);
   if (K < 8 || K % 8) return tis_fail("gemm_skinny: K=%d must be a multiple of 8", K);
   if (n_heads < 1 || n_kv_heads < 1 || head_dim < 4 || head_dim % 4 || page_size < 1)
     return tis_fail("gemm_skinny: heads=%d kv_heads=%d head_dim=%d (a multiple of 4) page=%d", n_heads, n_kv_heads,

@@ -97,6 +97,7 @@ def library(name: str) -> _Lib:
 
 # wavefronts the attention launch aims for, so that short batches still spread over the chip
 _SKINNY_MAX_ROWS = 32
+_SKINNY_MAX_ROWS_QKV = 64        # the q/k/v projection with norm, rotary and cache write fused stands for three launches
 _ATTN_TARGET_WAVES = 512
 _ATTN_PROMPT_TARGET_WAVES = 2048  # what the grid offers where rows of prompts are in the batch ...
 _ATTN_PROMPT_SPLIT_MAX_ROWS = 512 # ... and the batch is small; a long portion fills the chip by its rows alone
@@ -335,10 +336,10 @@ class HipOps:
             return out
         return self._linear_bf16(x, w, residual, out_dtype, reuse_residual)
 
-    def _skinny_ok(self, x, M, K):
+    def _skinny_ok(self, x, M, K, limit=None):
         # up to 32 rows the fused few-row kernel wins (it saves the norm, gating and rotary launches and streams the
         # weights as fast as the library does); beyond, the library's product is enough faster to pay for them
-        return (self.dtype == torch.bfloat16 and 0 < M <= _SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0
+        return (self.dtype == torch.bfloat16 and 0 < M <= (limit or _SKINNY_MAX_ROWS) and K % 8 == 0 and x.stride(0) % 8 == 0
                 and x.data_ptr() % 16 == 0)
 
     def linear_swiglu(self, x, w, rms=None):
@@ -418,7 +419,7 @@ class HipOps:
         N = (n_heads + 2 * n_kv_heads) * head_dim
         if w.dim() != 2 or tuple(w.shape) != (N, K) or not w.is_contiguous():
             raise KernelError(f"qkv_rope: w {tuple(w.shape)} is not [{N}, {K}] contiguous")
-        if self._skinny_ok(x, M, K) and head_dim % 4 == 0:
+        if self._skinny_ok(x, M, K, _SKINNY_MAX_ROWS_QKV) and head_dim % 4 == 0:
             self._index(positions, "positions", M)
             if table is not None:
                 self._check(table, "rotary table", torch.float32)

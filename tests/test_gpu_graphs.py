@@ -43,13 +43,16 @@ def test_graph_replays_match_eager_steps(name):
         assert (got[True][key] - got[False][key]).abs().max().item() <= 2 * tol, key
 
 
-def test_graph_survives_changing_batches():
-    """Requests join and leave: graphs of several shapes are captured and reused; results stay right."""
+@pytest.mark.parametrize("max_graphs", [32, 2])
+def test_graph_survives_changing_batches(max_graphs):
+    """Requests join and leave: graphs of several shapes are captured and reused; results stay right, also when
+    only two graphs may be kept and the least recently used one goes each time a third shape comes."""
     name = "D"
     folder = H.model_folder(name, "bfloat16")
     vocab = H.TINY[name]["cfg"].vocab_size
     reqs = {f"q{i}": H.random_ids(vocab, n, 60 + i) for i, n in enumerate([50, 30, 44, 38])}
     eng = Engine(folder, dtype="bfloat16", page_size=16, max_tokens=512, max_requests=8)
+    eng.max_graphs = max_graphs
     main = {}
     for rid, ids in reqs.items():
         eng.step([(rid, ids[:10], [])])
@@ -61,6 +64,6 @@ def test_graph_survives_changing_batches():
         for k, r in enumerate(live):
             main[(r, fed[r])] = lg[k]
             fed[r] += 1
-    assert len(eng._graphs) >= 3 and eng.graph_replays >= 30
+    assert min(3, max_graphs) <= len(eng._graphs) <= max_graphs and eng.graph_replays >= 30
     H.compare_with_plain(folder, reqs, main, {}, 2e-2 * max(1.0, max(
         H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values())), 0)

@@ -1,8 +1,8 @@
-// C[M,N] = f(A[M,K]) . W[N,K]^T for few rows (M <= 32): the matrix product of decode steps, where the job is to
-// stream W from HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950).
+// C[M,N] = f(A[M,K]) . W[N,K]^T for few rows (M <= 32; 64 for the q/k/v projection): the matrix product of decode
+// steps, where the job is to stream W from HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950).
 //
-// One workgroup owns 16 rows of W (16 output columns; 8 in the narrow variant below) over the whole of K; its waves take the 32-wide steps of
-// K in turn, so together they read each weight row in contiguous runs. W rows are the A operand straight from
+// One workgroup owns 16 rows of W (16 output columns; 8 in the narrow variant below) over the whole of K; its
+// waves take the 32-wide steps of K in turn, so together they read each weight row in contiguous runs. W rows are the A operand straight from
 // global memory (16 bytes per lane), the activations are the B operand straight from L2 (they are a few KB
 // and every workgroup reads the same ones), so no LDS is used for operands. Partial sums of the waves are
 // added through LDS in a fixed order: a row's result does not depend on M or on the other rows.
@@ -15,6 +15,8 @@
 //   RESIDUAL  C += R
 //   SWIGLU    W holds gate and up rows interleaved (gate_0, up_0, gate_1, ...): out[:, f] = silu(c[2f]) * c[2f+1]
 //             (main_models_new.py:51), written [M, N/2]
+//   ROPE      the q/k/v projection: rotary encoding of q and k by the row's position, q written out, k and v
+//             written into the row's cache slot (main_models_new.py:75-80, block_table.py:6-28); see RopeArgs
 // Output bfloat16 or float (the output table writes 32-bit logits).
 #include "common.h"
 

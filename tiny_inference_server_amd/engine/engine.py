@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import dataclasses
 from dataclasses import dataclass
+from collections import OrderedDict
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import torch
@@ -73,7 +74,8 @@ class Engine:
         # decode steps are replayed from captured graphs where the kernels allow it
         self.use_graphs = bool(use_graphs) and bool(getattr(ops, "supports_graphs", False)) and self.model.graph_safe
         self.graph_table_pages = 64          # block-table widths are rounded up to this many pages
-        self._graphs: Dict[Tuple[int, int], object] = {}
+        self._graphs: "OrderedDict[Tuple[int, int], object]" = OrderedDict()   # least recently used first
+        self.max_graphs = 32                 # each holds its step's activations; the oldest goes when there are more
         self._graph_seen: Dict[Tuple[int, int], int] = {}
         self.graph_replays = 0
 
@@ -184,6 +186,8 @@ class Engine:
         width = -(-pages // self.graph_table_pages) * self.graph_table_pages
         key = (len(batch_entries), width)
         graph = self._graphs.get(key)
+        if graph is not None:
+            self._graphs.move_to_end(key)
         if graph is not None and graph.slots == tuple(e.slot for e in batch_entries):
             for e in batch_entries:
                 if e.start + 1 > self.spec.max_context:
@@ -203,6 +207,9 @@ class Engine:
                     st.max_kv_len = width * self.page_size
                 outs = self.model.forward(step, self.cache)
                 return self.model.logits(outs[0].hidden, step.stages[0].want_index, len(batch_entries))
+            if len(self._graphs) >= self.max_graphs:
+                torch.cuda.synchronize(self.device)          # no replay of the graph to be dropped is still running
+                self._graphs.popitem(last=False)
             graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size)
         self.graph_replays += 1
         return graph.run(plan)

@@ -37,9 +37,12 @@ SOURCES: Dict[str, str] = {
     "attention_mfma": "attention_mfma.hip",
     "gemm_plain": "gemm_plain.hip",
     "gemm_skinny": "gemm_skinny.hip",
+    "gemm_library": "gemm_library.hip",
     "sampling": "sampling.hip",
 }
 HEADERS = ["common.h"]
+# what a library links beyond the HIP runtime
+LINK: Dict[str, List[str]] = {"gemm_library": ["-lhipblaslt"]}
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -93,7 +96,7 @@ def _digest(name: str) -> str:
     for f in [SOURCES[base]] + HEADERS:
         with open(os.path.join(CSRC, f), "rb") as fh:
             h.update(fh.read())
-    h.update(" ".join(FLAGS + defines).encode())
+    h.update(" ".join(FLAGS + defines + LINK.get(base, [])).encode())
     return h.hexdigest()[:12]
 
 
@@ -138,7 +141,7 @@ def _compile(name: str, out_dir: str) -> str:
     env = dict(os.environ)
     if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
         env["HOME"] = out_dir   # the compiler may want a cache folder
-    cmd = [_hipcc()] + FLAGS + defines + ["-I", CSRC, "-o", tmp, src]
+    cmd = [_hipcc()] + FLAGS + defines + ["-I", CSRC, "-o", tmp, src] + LINK.get(base, [])
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
     if proc.returncode != 0:
         try:

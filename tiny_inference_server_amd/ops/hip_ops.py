@@ -78,6 +78,10 @@ _SIGNATURES["gemm_skinny"] = ("tis_gemm_skinny", {
     "tis_gemm_skinny": [_P, _L, _P, _P, _F, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P],
     "tis_gemm_skinny_qkv_rope": [_P, _L, _P, _P, _F, _P, _L, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
 })
+_SIGNATURES["gemm_library"] = ("tis_gemm_library", {
+    "tis_gemm_library_init": [],
+    "tis_gemm_library": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _P],
+})
 _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
     "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I,
                            _P, _P],
@@ -155,13 +159,18 @@ class HipOps:
         self.code = _DT[dtype]
         # whatever is not built yet is compiled side by side, not one after the other
         _build.build(["rowwise", "rope_cache", "attention_generic", "gemm_plain", "sampling"] +
-                     (["gemm_skinny"] if dtype == torch.bfloat16 else []))
+                     (["gemm_skinny", "gemm_library"] if dtype == torch.bfloat16 else []))
         self.rowwise = library("rowwise")
         self.rope = library("rope_cache")
         self.attn_generic = library("attention_generic")
         self.gemm_plain = library("gemm_plain")
         self.sampling = library("sampling")
         self.gemm_skinny = library("gemm_skinny") if dtype == torch.bfloat16 else None
+        self.gemm_library = None
+        if dtype == torch.bfloat16:
+            self.gemm_library = library("gemm_library")
+            with torch.cuda.device(self.device):
+                self.gemm_library.tis_gemm_library_init()
         self._attn_groups = set()          # group sizes of the attention mixers built on these ops
         self._attn_mfma = {}               # head size -> library
         self._workspace = None
@@ -361,16 +370,22 @@ class HipOps:
         return self.swiglu(self.linear(x, w, rms=rms))
 
     def _linear_bf16(self, x, w, residual, out_dtype, reuse_residual=False):
+        """The library's product for many rows (reference main_models_new.py:19-20 uses one too)."""
+        M, K = x.shape
+        N = w.shape[0]
         if out_dtype == torch.float32:
             out = torch.matmul(x, w.t()).float()
             if residual is not None:
                 out += residual
             return out
-        if residual is not None:
-            if reuse_residual and residual.is_contiguous():
-                return torch.addmm(residual, x, w.t(), out=residual)
-            return torch.addmm(residual, x, w.t())
-        return torch.matmul(x, w.t())
+        if x.stride(0) % 8 or x.data_ptr() % 16 or (residual is not None and (residual.stride(0) % 8 or residual.data_ptr() % 16)):
+            # operands the library's fast kernels may not take as they lie: let the framework arrange them
+            return torch.addmm(residual, x, w.t()) if residual is not None else torch.matmul(x, w.t())
+        out = residual if (residual is not None and reuse_residual) else self.empty(M, N)
+        self.gemm_library.tis_gemm_library(_ptr(x), x.stride(0), _ptr(w), _ptr(residual),
+                                           residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0),
+                                           M, N, K, self._stream())
+        return out
 
     # ---- position encoding + cache write, attention --------------------------------------------------
     def rope_write_kv(self, qkv, positions, write_slots, table, plane, n_heads, n_kv_heads, head_dim, page_size,

@@ -155,6 +155,7 @@ class HipOps:
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: this engine runs on HIP kernels only and has no CPU path")
         self.device = torch.device(device)
+        self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         self.dtype = dtype
         self.code = _DT[dtype]
         # whatever is not built yet is compiled side by side, not one after the other
@@ -192,7 +193,9 @@ class HipOps:
 
     # ---- helpers -------------------------------------------------------------------------------------
     def _stream(self):
-        return c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        # torch's current stream of the device (under a graph capture: the capturing stream), by the short way:
+        # a kernel launch asks for it, and the public accessor builds a stream object each time (4 us)
+        return c_void_p(torch._C._cuda_getCurrentRawStream(self._device_index))
 
     def _check(self, t: torch.Tensor, what: str, dtype=None):
         dtype = dtype or self.dtype

@@ -261,3 +261,137 @@ def test_window_layers_get_pages_of_their_own_and_give_them_back(dtype, tol):
     eng.cache.check()
     assert all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups.values())
     ARCHITECTURES.unregister("WindowedToy")
+
+
+# ---- a toy feed-forward with routing and a toy position encoding, defined here, in the built-in block ------------
+
+from tiny_inference_server_amd.parts import FEED_FORWARDS, POSITION_ENCODINGS
+
+
+class ToyTop1Experts:
+    """Each row goes to the expert its router logit is largest for; y = p * expert(x), p being the softmax weight of
+    the chosen expert. Router logits and their softmax are 32-bit. An expert is a dense gated feed-forward."""
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        d, f, e = params["d_model"], params["hidden"], params["n_experts"]
+        shapes = {"router": (d, e)}
+        for i in range(e):
+            shapes.update({f"gate{i}": (d, f), f"up{i}": (d, f), f"down{i}": (f, d)})
+        return shapes
+
+    def __init__(self, spec, tensors, ops):
+        self.ops, self.n = ops, int(spec.params["n_experts"])
+        self.router = to_compute(ops, tensors.of(spec, "router").t())
+        self.gate_up, self.down = [], []
+        for i in range(self.n):
+            g, u = tensors.of(spec, f"gate{i}"), tensors.of(spec, f"up{i}")
+            self.gate_up.append(to_compute(ops, torch.stack((g.t(), u.t()), dim=1).reshape(2 * g.shape[1], g.shape[0])))
+            self.down.append(to_compute(ops, tensors.of(spec, f"down{i}").t()))
+
+    def forward(self, x, residual=None):
+        logits = self.ops.linear(x, self.router, out_dtype=torch.float32)
+        prob, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+        out = residual.clone() if residual is not None else torch.zeros_like(x)
+        for e in range(self.n):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                y = self.ops.linear(self.ops.linear_swiglu(x[rows].contiguous(), self.gate_up[e]), self.down[e])
+                out[rows] = (out[rows].float() + prob[rows, None] * y.float()).to(out.dtype)
+        return out
+
+
+class ToyStretchedRotary:
+    """Rotary encoding whose angle at position p is that of position p / stretch: another table, same kernels."""
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        return {}
+
+    def __init__(self, spec, tensors, ops):
+        p = spec.params
+        hd, self.max_context = int(p["head_dim"]), int(p["max_context"])
+        theta = 1.0 / torch.pow(torch.tensor(float(p["base"])), (2 * torch.arange(hd // 2).float()) / hd)
+        angle = torch.outer(torch.arange(self.max_context).float() / float(p["stretch"]), theta)
+        self.table = torch.stack((torch.cos(angle), torch.sin(angle)), dim=-1).contiguous().to(ops.device)
+
+    def rotary(self):
+        return self.table, False
+
+
+def routed_spec(cfg, n_experts, stretch):
+    from tiny_inference_server_amd.architectures.gqa_mtp import _block, _norm
+    import dataclasses
+    layers = []
+    for l in range(cfg.n_layers):
+        blk = _block(cfg, f"transformer_block_list.{l}.")
+        pos = PartSpec("position", "toy_stretched_rotary", {"head_dim": cfg.head_dim, "base": cfg.rope_base,
+                                                            "max_context": cfg.max_context, "stretch": stretch})
+        mixer = dataclasses.replace(blk.mixer, params={**blk.mixer.params, "position": pos})
+        names = {"router": f"l{l}.router"}
+        for e in range(n_experts):
+            names.update({f"gate{e}": f"l{l}.e{e}.g", f"up{e}": f"l{l}.e{e}.u", f"down{e}": f"l{l}.e{e}.d"})
+        ffn = PartSpec("feed_forward", "toy_top1_experts",
+                       {"d_model": cfg.d_model, "hidden": cfg.ffn_hidden, "n_experts": n_experts}, names)
+        # the second layer keeps the built-in dense feed-forward: parts are chosen layer by layer
+        layers.append(dataclasses.replace(blk, mixer=mixer, feed_forward=ffn if l != 1 else blk.feed_forward))
+    stage = StageSpec("trunk", 0, PartSpec("stage_input", "token_embedding"), tuple(LayerCall(l) for l in range(cfg.n_layers)),
+                      _norm(cfg, "rms_out.scale"))
+    return ModelSpec(cfg.d_model, cfg.vocab_size, cfg.max_context, tuple(layers), (stage,), "embedding.weight", "embedding.weight")
+
+
+def routed_plain(ids, w, cfg, n_experts, stretch):
+    T, D, NH, G = len(ids), cfg.d_model, cfg.n_heads, cfg.group_size
+    KVH, hd = NH // G, D // NH
+    x = w["embedding.weight"][torch.tensor(ids)]
+    j = torch.arange(hd // 2, dtype=torch.float64)
+    angle = torch.outer(torch.arange(T, dtype=torch.float64) / stretch, cfg.rope_base ** (-2 * j / hd))
+    cos, sin = torch.cos(angle).repeat(1, 2).unsqueeze(1), torch.sin(angle).repeat(1, 2).unsqueeze(1)
+    rope = lambda t: t * cos + pm.rotate_half(t) * sin
+    for l in range(cfg.n_layers):
+        pre = f"transformer_block_list.{l}."
+        a = pm.rms_norm(x, w[pre + "att.rms_norm_att.scale"], cfg.rms_eps)
+        q = (a @ w[pre + "att.q_proj.weight"]).view(T, NH, hd)
+        k, v = (a @ w[pre + "att.kv_proj.weight"]).view(T, 2, KVH, hd).unbind(1)
+        x = x + pm.causal_gqa_attention(rope(q), rope(k), v, G).reshape(T, D) @ w[pre + "att.linear_proj.weight"]
+        f = pm.rms_norm(x, w[pre + "rms_norm_ffn.scale"], cfg.rms_eps)
+        if l == 1:
+            x = x + pm.swiglu_ffn(f, w[pre + "ffn.swig.linear1.weight"], w[pre + "ffn.swig.linear2.weight"], w[pre + "ffn.fc.weight"])
+            continue
+        prob, choice = torch.softmax(f @ w[f"l{l}.router"], dim=-1).max(dim=-1)
+        y = torch.stack([pm.swiglu_ffn(f[r], w[f"l{l}.e{int(choice[r])}.g"], w[f"l{l}.e{int(choice[r])}.u"],
+                                        w[f"l{l}.e{int(choice[r])}.d"]) for r in range(T)])
+        x = x + prob[:, None] * y
+    return pm.rms_norm(x, w["rms_out.scale"], cfg.rms_eps) @ w["embedding.weight"].T
+
+
+def test_toy_routed_feed_forward_and_toy_position_encoding_in_the_built_in_block():
+    """A feed-forward that routes rows to experts and a position encoding with another table are registered from
+    here and used inside the framework's own block and attention mixer, layer by layer beside the built-in dense
+    feed-forward; whole prompts, portions and mixed steps give the plain model's logits."""
+    from tiny_inference_server_amd.config import GqaMtpConfig
+    FEED_FORWARDS.register("toy_top1_experts", ToyTop1Experts, replace=True)
+    POSITION_ENCODINGS.register("toy_stretched_rotary", ToyStretchedRotary, replace=True)
+    n_experts, stretch = 3, 2.5
+    cfg = GqaMtpConfig(d_model=96, vocab_size=157, max_context=256, rope_base=1e4, n_heads=6, n_layers=3, ffn_hidden=72,
+                       group_size=3, mtp_heads=0, architecture="RoutedToy")
+    ARCHITECTURES.register("RoutedToy", Architecture("RoutedToy", GqaMtpConfig, lambda c: routed_spec(c, n_experts, stretch)),
+                           replace=True)
+    w = random_tensors(cfg, 31, std=0.1, gain_jitter=0.1, dtype="float32")
+    eng = Engine(config=cfg, tensors=w, dtype="float32", page_size=16, max_tokens=256, max_requests=3)
+    assert not eng.use_graphs                       # the routed part made no promise about graph capture
+    w64 = {k: v.double() for k, v in w.items()}
+    reqs = {"a": H.random_ids(157, 45, 3), "b": H.random_ids(157, 18, 4)}
+    used = set()
+    for trace in (H.whole_trace(reqs), H.mixed_trace(reqs, 2, 5)[0], H.portions_trace({"a": reqs["a"]}, 7)):
+        got, _ = H.run_trace(eng, trace, heads=False)
+        for (rid, p), lg in got.items():
+            want = routed_plain(reqs[rid], w64, cfg, n_experts, stretch)[p]
+            assert (lg.double() - want).abs().max() <= 2e-5 * max(1.0, want.abs().max()), (rid, p)
+    for l in (0, 2):          # the routing is not trivial: more than one expert is chosen in a prompt
+        f = pm.rms_norm(w64["embedding.weight"][torch.tensor(reqs["a"])], w64[f"transformer_block_list.{l}.rms_norm_ffn.scale"], cfg.rms_eps)
+        used.add(len(set((f @ w64[f"l{l}.router"]).argmax(-1).tolist())))
+    assert max(used) > 1
+    ARCHITECTURES.unregister("RoutedToy")
+    FEED_FORWARDS.unregister("toy_top1_experts")
+    POSITION_ENCODINGS.unregister("toy_stretched_rotary")

@@ -12,8 +12,7 @@ every part class
 
 norm            __call__(x) -> y                       rows in, rows out
 position        rotary() -> (table | None, interleaved)   a table of (cos, sin) per position and pair for
-                                                       mixers that rotate queries and keys; and
-                on_embedding(x, batch) -> x            a hook for encodings that act on the embedded rows
+                                                       mixers that rotate queries and keys
 every part      graph_safe = True                      class attribute, only if what the part launches depends on the
                                                        step's device arrays alone (then decode steps may be captured
                                                        as graphs); absent or False keeps the model on plain launches

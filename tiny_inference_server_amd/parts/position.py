@@ -37,8 +37,6 @@ class Rotary:
     def rotary(self):
         return self.table, self.interleaved
 
-    def on_embedding(self, x, batch):
-        return x
 
 
 @POSITION_ENCODINGS.register("none")
@@ -55,5 +53,3 @@ class NoPosition:
     def rotary(self):
         return None, False
 
-    def on_embedding(self, x, batch):
-        return x

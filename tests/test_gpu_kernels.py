@@ -357,6 +357,9 @@ def test_product_with_norm_residual_and_gate_for_many_rows(ops_for, M, N, K):
     torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), xn @ w.double().t(), **t)
     torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), residual=res.cuda()).cpu().double(),
                                x.double() @ w.double().t() + res.double(), **t)
+    lg = ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32)          # the output table's case: 32-bit sums kept
+    assert lg.dtype == torch.float32 and ops._library_f32_out
+    torch.testing.assert_close(lg.cpu().double(), x.double() @ w.double().t(), rtol=1e-4, atol=1e-4)
     gu = (xn @ w.double().t()).to(torch.bfloat16).double()
     want = torch.nn.functional.silu(gu[:, 0::2]) * gu[:, 1::2]
     torch.testing.assert_close(ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), want,

@@ -30,8 +30,8 @@ struct Plan {
 struct DeviceState {
   hipblasLtHandle_t handle = nullptr;
   void* workspace = nullptr;
-  // (M, N, K, x_ld, r_ld or 0, c_ld)
-  std::map<std::tuple<int, int, int, long, long, long>, Plan> plans;
+  // (M, N, K, x_ld, r_ld or 0, c_ld, 32-bit output)
+  std::map<std::tuple<int, int, int, long, long, long, int>, Plan> plans;
 };
 
 constexpr size_t kWorkspaceBytes = 32u << 20;   // what the library may use for split reductions
@@ -64,15 +64,18 @@ TIS_EXPORT int tis_gemm_library_init() {
 
 // R: null, or the residual added to the product (it may be C itself). A shape's first call asks the library for
 // an algorithm and must not happen under stream capture; later calls only launch.
+// out_f32: C holds 32-bit floats (the output table's logits); no residual then.
 TIS_EXPORT int tis_gemm_library(const void* X, long x_ld, const void* W, const void* R, long r_ld, void* C, long c_ld,
-                                int M, int N, int K, hipStream_t stream) {
+                                int M, int N, int K, int out_f32, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (M < 0 || N < 0 || K < 1) return tis_fail("gemm_library: bad size M=%d N=%d K=%d", M, N, K);
   if (x_ld < K || c_ld < N || (R && r_ld < N)) return tis_fail("gemm_library: a row stride is shorter than its row");
+  if (out_f32 && R) return tis_fail("gemm_library: a 32-bit result takes no residual");
+  const hipDataType out_type = out_f32 ? HIP_R_32F : HIP_R_16BF;
   std::lock_guard<std::mutex> lock(g_mutex);
   DeviceState* st;
   if (device_state(&st)) return -1;
-  const auto key = std::make_tuple(M, N, K, x_ld, R ? r_ld : 0L, c_ld);
+  const auto key = std::make_tuple(M, N, K, x_ld, R ? r_ld : 0L, c_ld, out_f32 ? 1 : 0);
   auto it = st->plans.find(key);
   if (it == st->plans.end()) {
     Plan p;
@@ -82,8 +85,8 @@ TIS_EXPORT int tis_gemm_library(const void* X, long x_ld, const void* W, const v
     ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain)) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatrixLayoutCreate(&p.w, HIP_R_16BF, K, N, K) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatrixLayoutCreate(&p.x, HIP_R_16BF, K, M, x_ld) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && hipblasLtMatrixLayoutCreate(&p.r, HIP_R_16BF, N, M, R ? r_ld : c_ld) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && hipblasLtMatrixLayoutCreate(&p.c, HIP_R_16BF, N, M, c_ld) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatrixLayoutCreate(&p.r, out_type, N, M, R ? r_ld : c_ld) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatrixLayoutCreate(&p.c, out_type, N, M, c_ld) == HIPBLAS_STATUS_SUCCESS;
     if (!ok) return tis_fail("gemm_library: the library refused the descriptors of M=%d N=%d K=%d", M, N, K);
     hipblasLtMatmulPreference_t pref;
     if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return tis_fail("gemm_library: no preference object");

@@ -80,7 +80,7 @@ _SIGNATURES["gemm_skinny"] = ("tis_gemm_skinny", {
 })
 _SIGNATURES["gemm_library"] = ("tis_gemm_library", {
     "tis_gemm_library_init": [],
-    "tis_gemm_library": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _P],
+    "tis_gemm_library": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _I, _P],
 })
 _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
     "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I,
@@ -168,6 +168,7 @@ class HipOps:
         self.sampling = library("sampling")
         self.gemm_skinny = library("gemm_skinny") if dtype == torch.bfloat16 else None
         self.gemm_library = None
+        self._library_f32_out = True
         if dtype == torch.bfloat16:
             self.gemm_library = library("gemm_library")
             with torch.cuda.device(self.device):
@@ -376,18 +377,28 @@ class HipOps:
         """The library's product for many rows (reference main_models_new.py:19-20 uses one too)."""
         M, K = x.shape
         N = w.shape[0]
+        aligned = not (x.stride(0) % 8 or x.data_ptr() % 16 or
+                       (residual is not None and (residual.stride(0) % 8 or residual.data_ptr() % 16)))
         if out_dtype == torch.float32:
+            if aligned and residual is None and self._library_f32_out:
+                out = self.empty(M, N, dtype=torch.float32)      # 32-bit sums written as they are, not via bfloat16
+                try:
+                    self.gemm_library.tis_gemm_library(_ptr(x), x.stride(0), _ptr(w), _ptr(None), 0, _ptr(out), N, M, N,
+                                                       K, 1, self._stream())
+                    return out
+                except KernelError:
+                    self._library_f32_out = False       # a library without such kernels: round through bfloat16 below
             out = torch.matmul(x, w.t()).float()
             if residual is not None:
                 out += residual
             return out
-        if x.stride(0) % 8 or x.data_ptr() % 16 or (residual is not None and (residual.stride(0) % 8 or residual.data_ptr() % 16)):
+        if not aligned:
             # operands the library's fast kernels may not take as they lie: let the framework arrange them
             return torch.addmm(residual, x, w.t()) if residual is not None else torch.matmul(x, w.t())
         out = residual if (residual is not None and reuse_residual) else self.empty(M, N)
         self.gemm_library.tis_gemm_library(_ptr(x), x.stride(0), _ptr(w), _ptr(residual),
                                            residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0),
-                                           M, N, K, self._stream())
+                                           M, N, K, 0, self._stream())
         return out
 
     # ---- position encoding + cache write, attention --------------------------------------------------

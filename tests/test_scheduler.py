@@ -159,3 +159,39 @@ def test_uniform_stream():
 
 def test_pages_for():
     assert [pages_for(n, 16) for n in (0, 1, 16, 17)] == [0, 1, 1, 2]
+
+
+@pytest.mark.parametrize("static", ["req", 64, "ctx"])
+def test_static_modes_take_pages_at_admission_and_give_the_same_tokens(greedy_truth, static):
+    """The reference's storage policy static="ctx"/"req"/<int> (server.py:107-111, 151-166, 180-185): every page of
+    a request is taken when it is admitted, nothing is preempted, the tokens are the paged ones."""
+    eng = engine(16 * 64, max_requests=4)
+    s = Scheduler(eng, max_batch=4, token_budget=64, plan="cur", static=static,
+                  max_context=128 if static == "ctx" else None)
+    reqs = [Request(p, SamplingParams(max_new_tokens=20, temperature=0.0)) for p in prompts()]
+    for r in reqs:
+        s.submit(r)
+    s.admit()
+    want_pages = {"req": lambda r: pages_for(r.prompt_len + 20, 16), 64: lambda r: 4, "ctx": lambda r: 8}[static]
+    assert s.active and all(r.reserved == want_pages(r) * 16 for r in s.active)
+    assert eng.total_pages() - eng.free_pages() == sum(want_pages(r) for r in s.active)       # taken before any step
+    s.run()
+    assert [r.out_ids() for r in reqs] == greedy_truth
+    assert s.preempts == 0 and eng.free_pages() == eng.total_pages() and eng.cache.n_live == 0
+
+
+def test_static_reservation_larger_than_the_pool_is_an_error():
+    eng = engine(2 * 16, max_requests=2)
+    s = Scheduler(eng, max_batch=2, static=64)
+    s.submit(Request(prompts()[0], SamplingParams(max_new_tokens=4, temperature=0.0)))
+    with pytest.raises(RuntimeError, match="static reservation 4 pages > pool 2"):
+        s.admit()
+
+
+def test_static_admission_waits_for_pages_instead_of_preempting(greedy_truth):
+    """Six pages, every request reserves two or three: they run two at a time, and none is thrown out."""
+    eng = engine(6 * 16, max_requests=4)
+    out, s = generate(eng, prompts(), max_new_tokens=20, temperature=0.0, max_batch=4, plan="cur", static="req",
+                      return_scheduler=True)
+    assert out == greedy_truth and s.preempts == 0 and s.peak_running <= 3
+    assert eng.free_pages() == eng.total_pages() == 6

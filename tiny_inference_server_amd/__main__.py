@@ -64,6 +64,9 @@ def main(argv=None) -> int:
     ap.add_argument("--tokens-per-block", type=int, default=16)
     ap.add_argument("--token-budget", type=int, default=2048, help="most tokens one step runs")
     ap.add_argument("--plan", choices=["final", "cur"], default="final")
+    ap.add_argument("--static", default=None, metavar="MODE",
+                    help="take a request's pages at admission: 'ctx' (whole context), 'req' (prompt + new tokens) or a "
+                         "number of tokens; default: pages on demand")
     ap.add_argument("--heads", action="store_true",
                     help="also run the multi-token-prediction heads at every step (their drafts are not used)")
     a = ap.parse_args(argv)
@@ -104,7 +107,8 @@ def main(argv=None) -> int:
                            temperature=0.0 if a.greedy else a.temperature, top_k=0 if a.greedy else a.top_k,
                            top_p=0.0 if a.greedy else a.top_p, rep_penalty=1.0 if a.greedy else a.rep_penalty,
                            seed=a.seed, ignore_eos=a.ignore_eos, max_batch=a.max_batch, token_budget=a.token_budget,
-                           plan=a.plan, return_scheduler=True)
+                           plan=a.plan, static=(int(a.static) if a.static and a.static.isdigit() else a.static),
+                           return_scheduler=True)
     torch.cuda.synchronize()
     dt = time.time() - t0
     total = sum(len(o) for o in outs)

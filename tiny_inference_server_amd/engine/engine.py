@@ -89,6 +89,21 @@ class Engine:
         slot, _ = self.requests.pop(rid)
         self.cache.close_request(slot)
 
+    def reserve(self, rid: Hashable, n_tokens: int) -> None:
+        """Take now every page that `rid` needs to hold `n_tokens` positions (opening it if it is not live), the way
+        the reference's static storage modes do at admission (server.py:163-166). All or nothing: OutOfPages."""
+        opened = rid not in self.requests
+        if opened:
+            self.open(rid)
+        slot, _ = self.requests[rid]
+        n_tokens = min(int(n_tokens), self.spec.max_context)
+        if not self.cache.can_grow({slot: n_tokens}):
+            if opened:
+                self.close(rid)
+            raise OutOfPages(f"the cache cannot reserve {n_tokens} positions for request {rid!r}: free are "
+                             f"{self.cache.free_pages()}")
+        self.cache.grow(slot, n_tokens)
+
     def fed(self, rid: Hashable) -> int:
         return self.requests[rid][1]
 

@@ -13,13 +13,14 @@ def generate(model, prompts: Sequence[Sequence[int]], max_new_tokens: int = 200,
              dtype: str = "bfloat16", device: str = "cuda:0", max_batch: int = 8, token_budget: int = 2048,
              plan: str = "final", tokens_per_block: int = 16, pool_tokens: Optional[int] = None,
              params: Optional[Sequence[SamplingParams]] = None, return_scheduler: bool = False,
-             run_heads: bool = False):
+             run_heads: bool = False, static=None):
     """Generate for every prompt and return the new tokens, in the prompts' order.
 
     model: a model folder (config.json, model.safetensors) or an Engine already built. Request `i` draws from
     the random stream seed + i. pool_tokens: tokens the cache holds (default: room for max_batch full requests).
     run_heads: also run the multi-token-prediction heads at every step; their drafts are not used here, so by
     default generation runs the trunk alone (the reference's spec=False, server.py:106-118).
+    static: None (pages on demand), "ctx", "req" or a number of tokens: pages taken at admission (server.py:107-111).
     """
     if isinstance(model, Engine):
         engine = model
@@ -29,7 +30,7 @@ def generate(model, prompts: Sequence[Sequence[int]], max_new_tokens: int = 200,
             pool_tokens = max_batch * (-(-longest // tokens_per_block) * tokens_per_block)
         engine = Engine(model, dtype=dtype, page_size=tokens_per_block, max_tokens=pool_tokens,
                         max_requests=max_batch, device=device, run_heads=run_heads)
-    sched = Scheduler(engine, max_batch=max_batch, token_budget=token_budget, plan=plan)
+    sched = Scheduler(engine, max_batch=max_batch, token_budget=token_budget, plan=plan, static=static)
     reqs = []
     for i, p in enumerate(prompts):
         sp = params[i] if params is not None else SamplingParams(

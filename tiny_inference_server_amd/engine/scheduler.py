@@ -38,6 +38,7 @@ class Request:
         self.prompt_len = len(self.ids)
         self.params = params or SamplingParams(**kw)
         self.fed = 0            # positions whose keys and values are in the cache
+        self.reserved = 0       # positions whose pages a static mode took at admission
         self.done = False
         self.preempted = 0
 
@@ -61,9 +62,14 @@ def pages_for(n_tokens: int, page_size: int) -> int:
 
 class Scheduler:
     def __init__(self, engine, max_batch: int = 8, token_budget: int = 2048, plan: str = "final",
-                 max_context: Optional[int] = None):
+                 max_context: Optional[int] = None, static=None):
+        """static: how pages are taken (reference server.py:107-111). None: on demand, as the request grows.
+        "ctx": at admission, for the whole context; "req": for prompt plus max_new_tokens; an int: for that many
+        tokens. A request with a reservation never has to be preempted for pages it already holds."""
         if plan not in ("final", "cur"):
             raise ValueError(f"plan {plan!r}: use 'final' or 'cur'")
+        if not (static is None or static in ("ctx", "req") or (isinstance(static, int) and static > 0)):
+            raise ValueError(f"static {static!r}: use None, 'ctx', 'req' or a number of tokens")
         if max_batch < 1:
             raise ValueError(f"max_batch must be at least 1, got {max_batch}")
         if token_budget < max_batch:
@@ -72,6 +78,7 @@ class Scheduler:
         self.max_batch = min(max_batch, engine.cache.max_requests)
         self.token_budget = token_budget
         self.plan = plan
+        self.static = static
         self.max_context = min(max_context or engine.spec.max_context, engine.spec.max_context)
         self.eos = engine.spec.eos_token_id
         self.page_size = engine.page_size
@@ -92,11 +99,20 @@ class Scheduler:
         self.queue.append(req)
 
     def _held(self, r: Request) -> int:
-        return pages_for(r.fed, self.page_size) if r.fed else 0
+        tokens = max(r.fed, r.reserved)
+        return pages_for(tokens, self.page_size) if tokens else 0
 
     def _grow_pages(self, r: Request, n_new: int) -> int:
         """Pages r must take to be fed n_new more tokens."""
-        return pages_for(r.fed + n_new, self.page_size) - self._held(r)
+        return max(0, pages_for(r.fed + n_new, self.page_size) - self._held(r))
+
+    def _reserve_tokens(self, r: Request) -> int:
+        """Tokens a static mode reserves at admission (reference server.py:180-185)."""
+        if self.static == "ctx":
+            return self.max_context
+        if self.static == "req":
+            return min(r.prompt_len + r.params.max_new_tokens, self.max_context)
+        return min(int(self.static), self.max_context)
 
     def _final_pages(self, r: Request) -> int:
         """Pages r holds once it has generated all it may (the last token is sampled, never fed)."""
@@ -109,16 +125,23 @@ class Scheduler:
         budget = self.engine.free_pages() - sum(self._grow_pages(r, len(r.ids) - r.fed) for r in self.active)
         while self.queue and len(self.active) < self.max_batch:
             q = self.queue[0]
-            need_now = pages_for(len(q.ids), self.page_size)
-            if self.plan == "final":
+            need_now = pages_for(max(len(q.ids), self._reserve_tokens(q)) if self.static else len(q.ids), self.page_size)
+            if self.static and need_now > total:
+                raise RuntimeError(f"static reservation {need_now} pages > pool {total}")
+            if self.plan == "final" and not self.static:
                 projected = sum(self._final_pages(r) for r in self.active) + self._final_pages(q)
                 if projected > total and self.active:
                     break
-            elif need_now > budget and self.active:
+            elif need_now > budget and (self.active or self.static):
                 break
             budget -= need_now
             self.queue.popleft()
             q.fed = 0
+            q.reserved = 0
+            if self.static:
+                # every page now, so that this request never needs another (reference server.py:163-166)
+                q.reserved = need_now * self.page_size
+                self.engine.reserve(q.id, q.reserved)
             self.active.append(q)
 
     # ---- one step ------------------------------------------------------------------------------------
@@ -148,6 +171,7 @@ class Scheduler:
         if r.id in self.engine.requests:
             self.engine.close(r.id)
         r.fed = 0
+        r.reserved = 0
         r.preempted += 1
         self.queue.appendleft(r)
 

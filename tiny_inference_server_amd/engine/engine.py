@@ -11,6 +11,7 @@ from dataclasses import dataclass
 from collections import OrderedDict
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from .. import architectures  # noqa: F401  (registers the built-in architectures)
@@ -129,15 +130,18 @@ class Engine:
         if not entries:
             raise ValueError("a step needs at least one entry")
         seen = set()
+        arrays = {}
         for rid, toks, _ in entries:
             if rid in seen:
                 raise ValueError(f"request {rid!r} appears twice in one step")
             seen.add(rid)
             if len(toks) == 0:
                 raise ValueError(f"request {rid!r} brings no tokens")
-            for t in toks:
-                if not (0 <= int(t) < self.spec.vocab_size):
-                    raise ValueError(f"token {t} of request {rid!r} is outside the vocabulary of {self.spec.vocab_size}")
+            arr = arrays[rid] = np.asarray(toks)
+            if arr.dtype.kind not in "iu" or int(arr.min()) < 0 or int(arr.max()) >= self.spec.vocab_size:
+                bad = [t for t in toks if not (isinstance(t, (int, np.integer)) and 0 <= int(t) < self.spec.vocab_size)]
+                raise ValueError(f"token {bad[0] if bad else toks[0]!r} of request {rid!r} is outside the vocabulary "
+                                 f"of {self.spec.vocab_size}")
         opened = []
         for rid, _, _ in entries:
             if rid not in self.requests:
@@ -157,7 +161,7 @@ class Engine:
         for rid, toks, want in entries:
             slot, fed = self.requests[rid]
             self.cache.grow(slot, fed + len(toks))
-            batch_entries.append(Entry(slot, fed, list(toks), list(want)))
+            batch_entries.append(Entry(slot, fed, arrays[rid], list(want)))
         logits = None
         if (self.use_graphs and not heads and
                 all(len(e.tokens) == 1 and e.start >= self.model.max_lag and list(e.want) == [0]

@@ -12,6 +12,7 @@ import ctypes
 from ctypes import c_float, c_int, c_long, c_void_p
 from typing import Optional
 
+import numpy as np
 import torch
 
 from . import build as _build
@@ -113,7 +114,8 @@ _ATTN_WORKSPACE_FLOATS = 16 << 20
 def attention_items(seq_rows, group_size: int):
     """Work items of the matrix-core attention kernel for the rows of one stage.
 
-    seq_rows: (first row, first position, rows) per request. Returns (column blocks per item, [(first row, rows)]):
+    seq_rows: (first row, first position, rows) per request. Returns (column blocks per item, int32 array of
+    (first row, rows) lines):
     an item holds consecutive rows of one request, rows * group_size <= 16 * blocks. When no request has more
     than one row the list is simply every row in order, which the kernel knows without being given a list.
     """
@@ -127,15 +129,21 @@ def attention_items(seq_rows, group_size: int):
         nb *= 2
     per_item = max(1, (16 * nb) // group_size)
     if single:
-        return nb, [(first, 1) for first, _, n in seq_rows if n]
-    items = []
+        return nb, np.asarray([(first, 1) for first, _, n in seq_rows if n], dtype=np.int32).reshape(-1, 2)
+    firsts, counts, keys = [], [], []
     for first, p0, n in seq_rows:
-        for r in range(0, n, per_item):
-            items.append((p0 + r + min(per_item, n - r), first + r, min(per_item, n - r)))
+        if n <= 0:
+            continue
+        r = np.arange(0, n, per_item, dtype=np.int64)
+        cnt = np.minimum(per_item, n - r)
+        firsts.append(first + r)
+        counts.append(cnt)
+        keys.append(p0 + r + cnt)
+    firsts, counts, keys = np.concatenate(firsts), np.concatenate(counts), np.concatenate(keys)
     # the items with the most keys first: under a causal mask the last rows of a prompt are the longest, and
     # started last they would run on alone while the rest of the chip idles
-    items.sort(key=lambda it: -it[0])
-    return nb, [(first, n) for _, first, n in items]
+    order = np.argsort(-keys, kind="stable")
+    return nb, np.stack((firsts[order], counts[order]), axis=1).astype(np.int32)
 
 
 def _rows_view(t: torch.Tensor, what: str):
@@ -188,8 +196,8 @@ class HipOps:
         if self.dtype == torch.bfloat16:
             for group in sorted(self._attn_groups):
                 nb, items = attention_items(seq_rows, group)
-                if nb <= 4 and items:
-                    plans[("attention_items", group)] = (add([v for it in items for v in it]), len(items), nb)
+                if nb <= 4 and len(items):
+                    plans[("attention_items", group)] = (add(items), len(items), nb)
         return plans
 
     # ---- helpers -------------------------------------------------------------------------------------
@@ -510,7 +518,7 @@ class HipOps:
             plan = batch.extras.get(("attention_items", group))
             if plan is None:        # a caller that did not plan (a kernel test): plan now
                 nb, host_items = attention_items(batch.seq_rows, group)
-                items = torch.tensor(host_items, dtype=torch.int32).reshape(-1).to(self.device)
+                items = torch.from_numpy(np.ascontiguousarray(host_items)).reshape(-1).to(self.device)
                 plan = (items, len(host_items), nb)
             items, n_items, nb = plan
             if batch.max_seq_rows <= 1 and n_items == n:

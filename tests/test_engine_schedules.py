@@ -138,3 +138,21 @@ def test_long_context_decoding_in_bfloat16():
     main, _ = H.run_trace(eng, steps, heads=False)
     assert eng.graph_replays >= 100
     H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0)
+
+
+@pytest.mark.parametrize("backend", backends())
+@pytest.mark.parametrize("seed", [11, 12, 13, 14])
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("D", "bfloat16")])
+def test_random_schedules(name, dtype, backend, seed):
+    """Request lengths, the number of live requests, where prompts end and how they are cut all drawn at random, on
+    a pool just large enough: whatever the schedule, the logits are the plain model's."""
+    import random
+    rng = random.Random(seed)
+    lengths = [rng.choice((1, 2, 3, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 80, 100)) for _ in range(rng.randint(5, 9))]
+    reqs = requests_for(name, lengths, seed=seed)
+    steps, peak = H.mixed_trace(reqs, max_live=rng.randint(1, 4), seed=seed, prompt_frac=rng.choice((0.0, 0.3, 0.7, 1.0)))
+    folder, eng = make_engine(name, dtype, backend, max_tokens=peak)
+    main, heads = H.run_trace(eng, steps)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()

@@ -432,6 +432,27 @@ def test_projection_with_rotary_and_cache_write(ops_for, dtype, M, n_heads, n_kv
         torch.testing.assert_close(got.double().view(M, n_heads, hd), q * c + rot * s, **t)
 
 
+@pytest.mark.parametrize("M", [1, 8, 16])
+def test_skinny_product_with_two_column_tiles_a_workgroup(ops_for, M):
+    """Very wide matrices give a workgroup two column tiles. Forced here at a small width that ends inside the
+    second tile, for the plain, the 32-bit and the normed and gated product."""
+    ops, ref = ops_for(torch.bfloat16), TorchOps(dtype=torch.bfloat16)
+    N, K = 138, 800
+    x, w = rnd((M, K), torch.bfloat16, 91, 2.0), rnd((N, K), torch.bfloat16, 92, K ** -0.5)
+    gain = 1 + 0.1 * rnd((K,), torch.float32, 93)
+    narrow = [ops.linear(x.cuda(), w.cuda()).cpu(), ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32).cpu(),
+              ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()]
+    ops.gemm_skinny.cdll.tis_gemm_skinny_wide_tiles(1)
+    try:
+        wide = [ops.linear(x.cuda(), w.cuda()).cpu(), ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32).cpu(),
+                ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()]
+    finally:
+        ops.gemm_skinny.cdll.tis_gemm_skinny_wide_tiles(256)
+    for a, b in zip(narrow, wide):
+        assert torch.equal(a, b)          # the same sums in the same order, only spread over workgroups differently
+    torch.testing.assert_close(wide[1].double(), x.double() @ w.double().t(), rtol=1e-4, atol=1e-4)
+
+
 def test_sampling_with_the_context_kept_on_the_device(ops_for):
     """The penalty's context as a byte table per request instead of a token list: same draws, and the kernel marks
     what it drew."""

@@ -53,37 +53,47 @@ struct RopeArgs {
 // q/k/v projection, where this kernel stands for three launches (norm, product, rotary with cache write: 12.9k
 // against 12.7k at batch 64, 11.5k against 11.1k at batch 48); four blocks are built for that one only.
 //
+// CT: column tiles of 16 a workgroup owns. Two where the matrix is so wide that half as many workgroups still fill
+// the chip: a wave then uses the activations it loaded (and normed) for twice as many weights.
+//
 // R: with 16 output columns per workgroup a matrix of 1536 rows gives 96 workgroups, and a compute unit draws
 // only about 24 GB/s, so the 160 idle units cost more than the product. For M <= 16/R rows a workgroup
 // therefore owns only 16/R columns and fills the 16 rows of the matrix operand with R different 32-wide chunks of
 // K for those columns; the activation operand holds the same R chunks side by side. Of the 16x16 result only
 // the R diagonal blocks (chunk r of the weights against chunk r of the activations) mean anything; they are
 // added up with the waves' partial sums. R times as many workgroups, each step covers 32 R of K.
-template <int MB, bool NORM, int EPI, typename TO, int GS_WAVES, int U, int R>
+template <int MB, bool NORM, int EPI, typename TO, int GS_WAVES, int U, int R, int CT>
 __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
     const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const float* __restrict__ gain, float eps,
     const bf16* __restrict__ R_in, long r_ld, TO* __restrict__ C, long c_ld, int M, int N, int K, RopeArgs rope) {
   static_assert(MB == 1 || R == 1, "several row blocks go with full column tiles only");
+  static_assert(CT == 1 || (R == 1 && (EPI == EPI_NONE || EPI == EPI_SWIGLU)), "two column tiles: plain and gated products");
   constexpr int COLS = 16 / R;   // output columns of a workgroup, and the most rows of X a block takes
   constexpr int GH = 4 / R;      // lane groups of four result rows per chunk
-  __shared__ float red[GS_WAVES][MB][64][4];
+  __shared__ float red[GS_WAVES][MB][CT][64][4];
   __shared__ float red_ss[GS_WAVES][MB][16];
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
   const int chunk = c16 / COLS, sub = c16 % COLS;   // the lane's chunk of a step; its weight row and its activation row
-  const int n0 = blockIdx.x * COLS;
+  const int n0 = blockIdx.x * COLS * CT;
   const int steps = (K + 32 * R - 1) / (32 * R);
-  const bool w_ok = n0 + sub < N;
-  const bf16* wrow = W + (long)(w_ok ? n0 + sub : 0) * K + chunk * 32 + g * 8;
+  bool w_ok[CT];
+  const bf16* wrow[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    w_ok[ct] = n0 + ct * 16 + sub < N;
+    wrow[ct] = W + (long)(w_ok[ct] ? n0 + ct * 16 + sub : 0) * K + chunk * 32 + g * 8;
+  }
   bool x_ok[MB];
   const bf16* xrow[MB];
-  f32x4 acc[MB];
+  f32x4 acc[MB][CT];
   float ss[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     x_ok[mb] = mb * 16 + sub < M;
     xrow[mb] = X + (long)(x_ok[mb] ? mb * 16 + sub : 0) * x_ld + chunk * 32 + g * 8;
-    acc[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc[mb][ct] = (f32x4){0.f, 0.f, 0.f, 0.f};
     ss[mb] = 0.f;
   }
 
@@ -123,7 +133,7 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
   // U steps at a time: all their loads are issued before the first product, so that a wave keeps several
   // rows' worth of HBM requests in flight
   for (int s0 = wave; s0 < steps; s0 += U * GS_WAVES) {
-    bf16x8 a[U];
+    bf16x8 a[U][CT];
     bf16x8 b[U][MB];
     float gv[U][8];
 #pragma unroll
@@ -131,8 +141,11 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
       const int s = s0 + u * GS_WAVES;
       const int k = s * (32 * R) + chunk * 32 + g * 8;
       const bool k_ok = s < steps && k < K;   // K is a multiple of 8, so a lane's 8 values are all inside or all outside
-      a[u] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-      if (w_ok && k_ok) a[u] = *reinterpret_cast<const bf16x8*>(wrow + (long)s * (32 * R));
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        a[u][ct] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+        if (w_ok[ct] && k_ok) a[u][ct] = *reinterpret_cast<const bf16x8*>(wrow[ct] + (long)s * (32 * R));
+      }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         b[u][mb] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
@@ -158,7 +171,9 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
             bv[e] = static_cast<__bf16>(xf * gv[u][e]);
           }
         }
-        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc[mb], 0, 0, 0);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          acc[mb][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][ct], bv, acc[mb][ct], 0, 0, 0);
       }
     }
   }
@@ -167,7 +182,9 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][mb][lane][i] = acc[mb][i];
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][mb][ct][lane][i] = acc[mb][ct][i];
     if (NORM) {
       float t = ss[mb];
       t += __shfl_xor(t, 16, 64);
@@ -180,9 +197,10 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
   // result lane (gh, c): columns n0 + 4 gh + i of the rows mb * 16 + c; chunk r's share sits with lane (r GH + gh, r COLS + c)
   const int gh = lane >> 4, c = lane & 15;
   if (gh >= GH || c >= COLS) return;
-  const int n = n0 + gh * 4;   // the lane's four consecutive output columns
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
+  for (int mbct = 0; mbct < MB * CT; ++mbct) {
+    const int mb = mbct / CT, ct = mbct % CT;
+    const int n = n0 + ct * 16 + gh * 4;   // the lane's four consecutive output columns
     const int m = mb * 16 + c;
     if (m >= M) continue;
     float v[4];
@@ -193,7 +211,7 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
       for (int r = 0; r < R; ++r) {
         const int src = (r * GH + gh) * 16 + r * COLS + c;
 #pragma unroll
-        for (int w = 0; w < GS_WAVES; ++w) t += red[w][mb][src][i];
+        for (int w = 0; w < GS_WAVES; ++w) t += red[w][mb][ct][src][i];
       }
       v[i] = t;
     }
@@ -267,6 +285,8 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
 
 // A hook for tuning runs: forces (waves, U, R) for every launch of this process; zeros give the choice back.
 static int g_force_waves = 0, g_force_u = 0, g_force_r = 0;
+static int g_wide_tiles = 256;   // from this many 32-column workgroups on (one a compute unit), a workgroup takes two column tiles
+TIS_EXPORT void tis_gemm_skinny_wide_tiles(int n_workgroups) { g_wide_tiles = n_workgroups; }
 TIS_EXPORT void tis_gemm_skinny_force_config(int waves, int u, int r) {
   g_force_waves = waves;
   g_force_u = u;
@@ -297,11 +317,30 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
   }
   if (g_force_waves) { waves = g_force_waves; u = g_force_u; }
   if (mb > 1 && waves != 8) { waves = 8; u = 4; }   // several row blocks are built for eight waves only
-  const int cols = 16 / r;
+  // two column tiles a workgroup where the matrix is wide enough to fill the chip with half as many workgroups:
+  // the activations, the gains and the norm's arithmetic are then shared by twice as many weights (the gate-up
+  // product of 8192 columns and the output table: 2.5 % of a decode step at batch 8)
+  int ct = 1;
+  if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) {
+    if (r == 1 && mb == 1 && waves == 8 && (N + 31) / 32 >= g_wide_tiles) ct = 2;
+  }
+  const int cols = 16 / r * ct;
   const int n_wg = (N + cols - 1) / cols;
+  if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) {
+    if (ct == 2 && u == 3) {
+      gemm_skinny_kernel<1, NORM, EPI, TO, 8, 3, 1, 2><<<n_wg, 8 * 64, 0, stream>>>(
+          (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);
+      return 0;
+    }
+    if (ct == 2 && u == 4) {
+      gemm_skinny_kernel<1, NORM, EPI, TO, 8, 4, 1, 2><<<n_wg, 8 * 64, 0, stream>>>(
+          (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);
+      return 0;
+    }
+  }
 #define CFG(MBV, WV, UV, RV)                                                                                     \
-  if (mb == MBV && waves == WV && u == UV && r == RV) {                                                          \
-    gemm_skinny_kernel<MBV, NORM, EPI, TO, WV, UV, RV><<<n_wg, WV * 64, 0, stream>>>(                            \
+  if (ct == 1 && mb == MBV && waves == WV && u == UV && r == RV) {                                               \
+    gemm_skinny_kernel<MBV, NORM, EPI, TO, WV, UV, RV, 1><<<n_wg, WV * 64, 0, stream>>>(                         \
         (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);     \
     return 0;                                                                                                    \
   }

@@ -286,7 +286,9 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
 // A hook for tuning runs: forces (waves, U, R) for every launch of this process; zeros give the choice back.
 static int g_force_waves = 0, g_force_u = 0, g_force_r = 0;
 static int g_wide_tiles = 256;   // from this many 32-column workgroups on (one a compute unit), a workgroup takes two column tiles
+static int g_wide_max_blocks = 2;   // with up to two blocks of 16 rows (four blocks measured no gain over the library)
 TIS_EXPORT void tis_gemm_skinny_wide_tiles(int n_workgroups) { g_wide_tiles = n_workgroups; }
+TIS_EXPORT void tis_gemm_skinny_wide_max_blocks(int n) { g_wide_max_blocks = n; }
 TIS_EXPORT void tis_gemm_skinny_force_config(int waves, int u, int r) {
   g_force_waves = waves;
   g_force_u = u;
@@ -322,21 +324,19 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
   // product of 8192 columns and the output table: 2.5 % of a decode step at batch 8)
   int ct = 1;
   if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) {
-    if (r == 1 && mb == 1 && waves == 8 && (N + 31) / 32 >= g_wide_tiles) ct = 2;
+    if (r == 1 && mb <= g_wide_max_blocks && waves == 8 && (N + 31) / 32 >= g_wide_tiles) ct = 2;
   }
   const int cols = 16 / r * ct;
   const int n_wg = (N + cols - 1) / cols;
   if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) {
-    if (ct == 2 && u == 3) {
-      gemm_skinny_kernel<1, NORM, EPI, TO, 8, 3, 1, 2><<<n_wg, 8 * 64, 0, stream>>>(
-          (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);
-      return 0;
-    }
-    if (ct == 2 && u == 4) {
-      gemm_skinny_kernel<1, NORM, EPI, TO, 8, 4, 1, 2><<<n_wg, 8 * 64, 0, stream>>>(
-          (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);
-      return 0;
-    }
+#define WIDE(MBV, UV)                                                                                            \
+  if (ct == 2 && mb == MBV && u == UV) {                                                                         \
+    gemm_skinny_kernel<MBV, NORM, EPI, TO, 8, UV, 1, 2><<<n_wg, 8 * 64, 0, stream>>>(                            \
+        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);     \
+    return 0;                                                                                                    \
+  }
+    WIDE(1, 3) WIDE(1, 4) WIDE(2, 3) WIDE(2, 4)
+#undef WIDE
   }
 #define CFG(MBV, WV, UV, RV)                                                                                     \
   if (ct == 1 && mb == MBV && waves == WV && u == UV && r == RV) {                                               \

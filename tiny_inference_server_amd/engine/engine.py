@@ -137,6 +137,12 @@ class Engine:
             seen.add(rid)
             if len(toks) == 0:
                 raise ValueError(f"request {rid!r} brings no tokens")
+            if len(toks) <= 16:          # a few decoded tokens: plain checks beat building an array
+                for t in toks:
+                    if not (0 <= int(t) < self.spec.vocab_size):
+                        raise ValueError(f"token {t} of request {rid!r} is outside the vocabulary of {self.spec.vocab_size}")
+                arrays[rid] = list(toks)
+                continue
             arr = arrays[rid] = np.asarray(toks)
             if arr.dtype.kind not in "iu" or int(arr.min()) < 0 or int(arr.max()) >= self.spec.vocab_size:
                 bad = [t for t in toks if not (isinstance(t, (int, np.integer)) and 0 <= int(t) < self.spec.vocab_size)]

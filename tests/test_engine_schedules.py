@@ -156,3 +156,18 @@ def test_random_schedules(name, dtype, backend, seed):
     H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
     eng.cache.check()
     assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.parametrize("backend", backends())
+@pytest.mark.parametrize("name,dtype", [("D", "bfloat16"), ("B", "float32")])
+def test_what_a_page_held_before_never_reaches_a_result(name, dtype, backend):
+    """Every page starts out full of NaN, as if a broken request had owned it: masked slots are read by the kernels
+    but must not enter their arithmetic, not even weighted by zero."""
+    lengths = [50, 64, 37, 90, 18, 70]
+    reqs = requests_for(name, lengths, seed=8)
+    steps, peak = H.mixed_trace(reqs, max_live=3, seed=9)
+    folder, eng = make_engine(name, dtype, backend, max_tokens=peak)
+    for g in eng.cache.groups.values():
+        g.storage.fill_(float("nan"))
+    main, heads = H.run_trace(eng, steps)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)

@@ -118,8 +118,8 @@ def make_paged(kv_lens, n_kv, hd, page_size, dtype, seed, shuffle=True):
     ids = list(range(n_pages))
     if shuffle:
         random.Random(seed).shuffle(ids)
-    # unused slots hold huge values: a kernel that reads a masked slot shows it
-    plane = torch.full((n_pages, 2, n_kv, page_size, hd), 3e4, dtype=dtype)
+    # unused slots hold NaN: a kernel that lets a masked slot into its arithmetic, even weighted by zero, shows it
+    plane = torch.full((n_pages, 2, n_kv, page_size, hd), float("nan"), dtype=dtype)
     tables, ks, vs = [], [], []
     width = max(-(-L // page_size) for L in kv_lens)
     for i, L in enumerate(kv_lens):

@@ -17,8 +17,9 @@
 //                                              bfloat16 (as the reference does before P.V:
 //                                              paged_attention_kernels.py:108), exactly as S^T left it in registers
 // Both products put the column on the lane, so the softmax statistics never cross lanes except for the
-// reduction over the four key groups, and no LDS is used. Masked keys are read but multiplied by an exact 0:
-// every value ever found in the pool must be finite, which the pool's one-time zeroing ensures.
+// reduction over the four key groups, and no LDS is used. Masked keys are read (their page is mapped), but their
+// scores are replaced by -inf and their values by zero before either is used in arithmetic, so what an earlier
+// owner left in a page never reaches a result.
 #include "common.h"
 
 #ifndef TIS_HD
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
       }
     }
   };
-  auto consume = [&](int s, const Tiles& T) {
+  auto consume = [&](int s, Tiles& T) {
     const int kb = k_lo + s * 32;
     // S^T = K . Q^T
     f32x4 st[2][NB];
@@ -178,6 +179,20 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     // A step whose 32 keys lie inside every column's range needs no mask at all (most steps of a long row).
     const bool full = T.ok[0] && T.ok[1] && kb + 31 <= p_first && kb >= lo_last;
     if (!full) {
+      // Values of keys that no column of the item may see (slots past its last position, keys before its window,
+      // tiles past its range) are set to zero and not merely weighted by zero: what lies there is whatever an
+      // earlier owner of the page left, possibly not even finite.
+      const int lo_first = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = kb + t * 16 + g * 4 + e;
+          if (!(T.ok[t] && key <= p_last && key >= lo_first)) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) T.v[db][t * 4 + e] = static_cast<__bf16>(0.f);
+          }
+        }
       // one branch a step around all the masking, not one around each score
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)

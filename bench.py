@@ -156,7 +156,7 @@ def main() -> int:
         # the reference's "plain" decode runs no prediction heads; the same here, for comparison with its numbers
         pts[f"decode_b{a.batch}_trunk_only"] = round(decode_rate(a.batch, a.steps, a.warmup, trunk)[0], 1)
     line = {
-        "metric": "decode tok/s at batch 8 (0.9B, bf16); prefill tok/s at 2,048 tokens",
+        "metric": f"decode tok/s at batch {a.batch} ({a.size}, {dkey}); prefill tok/s at {a.prefill_tokens:,} tokens",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(sec_per_step * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": round(value / REFERENCE_B8_TOKS, 2) if (a.batch == 8 and a.size == "0.9B") else None,

@@ -36,7 +36,7 @@ def rnd(shape, dtype, seed, scale=1.0):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("rows,D", [(1, 8), (7, 1536), (33, 1000), (3, 5000)])
+@pytest.mark.parametrize("rows,D", [(1, 8), (7, 1536), (33, 1000), (3, 5000), (70, 1536), (35, 4096), (33, 4104), (41, 64)])
 def test_rmsnorm(ops_for, dtype, rows, D):
     ops, ref = ops_for(dtype), TorchOps(dtype=dtype)
     x = rnd((rows, D), dtype, 1, 3.0)

@@ -1,0 +1,121 @@
+"""Times one kernel alone on synthetic operands, for profiling runs and for tuning.
+
+    python -m tiny_inference_server_amd.ops.kernel_bench attention --segments 0:2048
+    python -m tiny_inference_server_amd.ops.kernel_bench attention --segments 4095:1x8
+    python -m tiny_inference_server_amd.ops.kernel_bench product --rows 8 --out 8192 --in 1536 --kind norm+gate
+
+A segment is `first position:rows`, `xN` repeats it for N requests; `4095:1x8` is a decode step of 8 requests at
+context 4096, `0:2048` a prompt of 2,048 tokens, `4095:1x8,1000:256` a mixed step. The kernel is captured into a
+graph of `--reps` launches and the graph is timed, so host launch cost stays out. A kernel alone runs on warm caches:
+decisions about decode kernels are taken on whole decode steps (bench.py), this is for counters and first looks.
+"""
+from __future__ import annotations
+
+import argparse
+import sys
+from types import SimpleNamespace
+
+import torch
+
+
+def graph_time(fn, reps: int) -> float:
+    """Microseconds per call of `fn`, median of seven replays of a graph that holds `reps` calls."""
+    fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(reps):
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    times = []
+    for _ in range(7):
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b) * 1000 / reps)
+    return sorted(times)[3]
+
+
+def parse_segments(text: str):
+    segs = []
+    for part in text.split(","):
+        body, _, times = part.partition("x")
+        first, _, rows = body.partition(":")
+        segs += [(int(first), int(rows))] * (int(times) if times else 1)
+    return segs
+
+
+def attention_case(ops, a):
+    from .hip_ops import attention_items
+    nh, kvh, hd, ps = a.heads, a.kv_heads, a.head_dim, a.page_size
+    segs = parse_segments(a.segments)
+    pages = [-(-(p0 + n) // ps) for p0, n in segs]
+    plane = torch.randn(sum(pages) + 4, 2, kvh, ps, hd, device=ops.device).to(torch.bfloat16)
+    tables = torch.zeros(len(segs), max(pages), dtype=torch.int32)
+    positions, row_seq, seq_rows, nxt = [], [], [], 0
+    for i, ((p0, n), k) in enumerate(zip(segs, pages)):
+        tables[i, :k] = torch.arange(nxt, nxt + k)
+        nxt += k
+        seq_rows.append((len(positions), p0, n))
+        positions += list(range(p0, p0 + n))
+        row_seq += [i] * n
+    rows = len(positions)
+    q = torch.randn(rows, nh * hd, device=ops.device).to(torch.bfloat16)
+    batch = SimpleNamespace(positions=torch.tensor(positions, dtype=torch.int32, device=ops.device),
+                            row_seq=torch.tensor(row_seq, dtype=torch.int32, device=ops.device),
+                            block_tables={"g": tables.to(ops.device)}, max_kv_len=max(p0 + n for p0, n in segs),
+                            extras={}, n_rows=rows, max_seq_rows=max(n for _, n in segs), seq_rows=seq_rows)
+    nb, items = attention_items(seq_rows, nh // kvh)
+    batch.extras[("attention_items", nh // kvh)] = (torch.as_tensor(items, dtype=torch.int32).reshape(-1).to(ops.device),
+                                                    len(items), nb)
+    us = graph_time(lambda: ops.paged_attention(q, plane, batch, "g", nh, kvh, hd), a.reps)
+    kv_bytes = sum(p0 + n for p0, n in segs) * kvh * hd * 2 * 2
+    flops = sum(4 * nh * hd * (n * p0 + n * (n + 1) / 2) for p0, n in segs)
+    print(f"attention {a.segments}: {us:.1f} us; keys and values {kv_bytes / 1e6:.1f} MB -> {kv_bytes / us / 1e6:.2f} TB/s; "
+          f"{flops / us / 1e6:.1f} TFLOP/s")
+
+
+def product_case(ops, a):
+    m, n, k = a.rows, a.out, a.inner
+    x = torch.randn(m, k, device=ops.device).to(torch.bfloat16)
+    w = (torch.randn(n, k, device=ops.device) * k ** -0.5).to(torch.bfloat16)
+    res = torch.randn(m, n, device=ops.device).to(torch.bfloat16)
+    rms = (torch.ones(k, device=ops.device), 1e-6)
+    kinds = {"plain": lambda: ops.linear(x, w), "residual": lambda: ops.linear(x, w, residual=res),
+             "norm": lambda: ops.linear(x, w, rms=rms), "norm+gate": lambda: ops.linear_swiglu(x, w, rms=rms),
+             "logits": lambda: ops.linear(x, w, out_dtype=torch.float32)}
+    us = graph_time(kinds[a.kind], a.reps)
+    print(f"product {a.kind} rows {m} out {n} in {k}: {us:.2f} us; weights {n * k * 2 / 1e6:.1f} MB -> "
+          f"{n * k * 2 / us / 1e6:.2f} TB/s; {2 * m * n * k / us / 1e6:.1f} TFLOP/s")
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="python -m tiny_inference_server_amd.ops.kernel_bench", description=__doc__,
+                                 formatter_class=argparse.RawDescriptionHelpFormatter)
+    sub = ap.add_subparsers(dest="what", required=True)
+    at = sub.add_parser("attention")
+    at.add_argument("--segments", default="4095:1x8")
+    at.add_argument("--heads", type=int, default=12)
+    at.add_argument("--kv-heads", type=int, default=3)
+    at.add_argument("--head-dim", type=int, default=128)
+    at.add_argument("--page-size", type=int, default=16)
+    pr = sub.add_parser("product")
+    pr.add_argument("--rows", type=int, default=8)
+    pr.add_argument("--out", type=int, default=8192)
+    pr.add_argument("--in", dest="inner", type=int, default=1536)
+    pr.add_argument("--kind", choices=["plain", "residual", "norm", "norm+gate", "logits"], default="plain")
+    for p in (at, pr):
+        p.add_argument("--reps", type=int, default=20)
+        p.add_argument("--device", default="cuda:0")
+    a = ap.parse_args(argv)
+    from .hip_ops import HipOps
+    ops = HipOps(a.device, torch.bfloat16)
+    (attention_case if a.what == "attention" else product_case)(ops, a)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -251,6 +251,66 @@ def test_mixed_rows_with_key_splits_chosen_item_by_item(ops_for, n_heads, n_kv, 
         torch.testing.assert_close(got[r].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,page_size,window", [
+    (12, 3, 128, 16, 0), (12, 3, 128, 16, 100), (4, 4, 64, 16, 0), (6, 2, 48, 32, 0), (16, 2, 32, 48, 45),
+    (2, 1, 256, 16, 0), (5, 1, 16, 16, 33), (20, 1, 32, 16, 0)])
+def test_long_portions_by_tiles(ops_for, n_heads, n_kv, hd, page_size, window):
+    """Portions long enough for the workgroup kernel (tiles of rows whose four waves share each step's keys through
+    LDS), beside rows that stay with the one-wave kernel: a whole prompt that ends mid-tile and mid-page, a portion
+    deep into a long request (its tiles are cut into key splits and merged), a decoded token and a three-row portion.
+    Group sizes that divide a wave's 64 columns and ones that do not; heads wider than 128 have 32-column waves."""
+    from tiny_inference_server_amd.ops.hip_ops import attention_items, tile_columns
+    ops = ops_for(torch.bfloat16)
+    group = n_heads // n_kv
+    tile_rows = 4 * (tile_columns(hd) // group)
+    n0, n1 = 2 * tile_rows + tile_rows // 2 + 5, tile_rows + 3
+    kv_lens = [n0, 1000 + n1, 700, 12]
+    segs = [(0, 0, n0), (1, 1000, n1), (2, 699, 1), (3, 9, 3)]
+    plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page_size, torch.bfloat16, seed=36)
+    positions, row_seq, seq_rows = [], [], []
+    for s_, p0, n in segs:
+        seq_rows.append((len(positions), p0, n))
+        positions += list(range(p0, p0 + n)); row_seq += [s_] * n
+    R = len(positions)
+    _, items, tiles, _ = attention_items(seq_rows, group, tile_columns(hd))
+    short_too = 3 >= max(2, tile_rows // 2)
+    assert len(tiles) == -(-n0 // tile_rows) + -(-n1 // tile_rows) + short_too and len(items) >= 1   # both kernels run
+    q = rnd((R, n_heads * hd), torch.bfloat16, 37)
+    batch = SimpleNamespace(positions=torch.tensor(positions, dtype=torch.int32).cuda(),
+                            row_seq=torch.tensor(row_seq, dtype=torch.int32).cuda(),
+                            block_tables={"g": tables.cuda()}, max_kv_len=max(kv_lens), extras={},
+                            n_rows=R, max_seq_rows=n0, seq_rows=seq_rows)
+    got = ops.paged_attention(q.cuda(), plane.cuda(), batch, "g", n_heads, n_kv, hd, window=window).cpu()
+    assert torch.isfinite(got.float()).all()
+    step = max(1, R // 60)
+    for r in sorted(set(list(range(0, R, step)) + [0, 1, 15, 16, tile_rows - 1, tile_rows, n0 - 1, n0, n0 + 1, R - 5, R - 4, R - 1])):
+        want = dense_reference(q[r].view(n_heads, hd), ks[row_seq[r]], vs[row_seq[r]], group, positions[r], window)
+        torch.testing.assert_close(got[r].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
+
+
+def test_a_tile_sees_a_far_key_and_a_rows_own_key(ops_for):
+    """Two scores are made to stand out in a long portion: a key far back (in an early split of the tile's keys) for
+    one row, and for another row the key at its own position, the last one the causal mask lets through."""
+    ops = ops_for(torch.bfloat16)
+    n_heads, n_kv, hd, page_size, L = 4, 1, 64, 16, 1200
+    plane, tables, ks, vs = make_paged([L], n_kv, hd, page_size, torch.bfloat16, seed=38)
+    p0, n = 900, 300
+    q = rnd((n, n_heads * hd), torch.bfloat16, 39)
+    for row, key in ((250, 3), (250, 1150), (77, 977), (77, 978)):
+        k = ks[0].clone()
+        k[key, 0] = (q[row].view(n_heads, hd)[0] * 4).to(torch.bfloat16)
+        pl = plane.clone()
+        pl[tables[0, key // page_size].item(), 0, 0, key % page_size] = k[key, 0]
+        batch = SimpleNamespace(positions=torch.arange(p0, p0 + n, dtype=torch.int32).cuda(),
+                                row_seq=torch.zeros(n, dtype=torch.int32).cuda(), block_tables={"g": tables.cuda()},
+                                max_kv_len=L, extras={}, n_rows=n, max_seq_rows=n, seq_rows=[(0, p0, n)])
+        got = ops.paged_attention(q.cuda(), pl.cuda(), batch, "g", n_heads, n_kv, hd).cpu()
+        want = dense_reference(q[row].view(n_heads, hd), k, vs[0], n_heads, p0 + row)
+        torch.testing.assert_close(got[row].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
+        seen = key <= p0 + row
+        assert ((got[row].view(n_heads, hd)[0].double() - vs[0][key, 0].double()).abs().max() < 0.05) == seen
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_one_far_key_among_hundreds(ops_for, dtype):
     """One key far back is made to dominate: a kernel that skips a page or a split would miss it."""

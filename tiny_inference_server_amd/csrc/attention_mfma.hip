@@ -20,6 +20,8 @@
 // reduction over the four key groups, and no LDS is used. Masked keys are read (their page is mapped), but their
 // scores are replaced by -inf and their values by zero before either is used in arithmetic, so what an earlier
 // owner left in a page never reaches a result.
+#include <type_traits>
+
 #include "common.h"
 
 #ifndef TIS_HD
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ items,
     bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
     int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits, int min_steps,
-    int* __restrict__ row_splits) {
+    int split_stride, int* __restrict__ row_splits) {
   const int page_size = PS16 ? 16 : page_size_arg;
   const int item = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int lane = threadIdx.x, c16 = lane & 15, g = lane >> 4;
@@ -313,7 +315,378 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
         *reinterpret_cast<bf16x4*>(dst + db * 16) = w;
       }
     } else {
-      const long slot = ((long)col_row[nb] * n_heads + col_head[nb]) * n_splits + split;
+      const long slot = ((long)col_row[nb] * n_heads + col_head[nb]) * split_stride + split;
+      float* dst = part_o + slot * HD + g * 4;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + db * 16) = o[nb][db];
+      if (g == 0) part_ml[slot] = make_float2(m[nb], lt);
+    }
+  }
+}
+
+// ---- Long portions of prompts: a workgroup of four waves shares every step's keys and values through LDS ----
+//
+// A wave of the kernel above fetches its keys and values itself, so the rows of a prompt read each key once per
+// 16*NB columns, and a wave waits out the fetch of every step. Here a *tile* is up to TW * (16 * TNB / group size)
+// consecutive rows of one request; its four waves own 16 * TNB columns each and walk the tile's keys together. Each
+// step's 32 keys and values are copied once from the pages into LDS, two steps ahead of the products that read
+// them, by loads that write LDS directly (global_load_lds: no registers, no store instructions), and every wave takes
+// its operands from there. LDS holds them in the order the products read them: 16-byte pieces, the 64 pieces of one
+// operand fetch side by side, so that reads meet no bank conflict and need no padding; a copying lane picks the
+// piece of the page that belongs in its slot. The arithmetic of a step is the wave kernel's, in another order: the
+// scores of step s+1 are multiplied out (matrix cores) while the exponentials of step s are taken (vector unit), so
+// that a wave keeps both busy. (Heads wider than 128: 16 columns a wave.)
+static constexpr int TW = 4;               // waves of a tile
+static constexpr int TNB = HD > 128 ? 1 : 2;   // column blocks of a wave: what leaves registers for several waves a SIMD
+static constexpr int TBUF = 3;             // LDS buffers: step s+1's keys, step s's values, and step s+2 being written
+static constexpr int NCH = HD / 8;         // 16-byte pieces of one key
+static constexpr int TCH = 4 * HD;         // pieces of a step's keys, and of its values: HD / 16 fetches of 64
+static constexpr int TPT = (TCH + TW * 64 - 1) / (TW * 64);   // fetches a wave issues, of each
+// keys:   piece (t, dch, c16) = key t*16 + c16, elements dch*8.. at piece index (t*NCH + dch)*16 + c16
+// values: piece (t, db, gh, c16) = element db*16 + c16 of the head, keys t*16 + gh*8.. at ((t*DB + db)*2 + gh)*16 + c16
+
+#pragma clang diagnostic ignored "-Winline-asm"   // M0 in a clobber list: meant
+// One 16-byte piece per lane from global memory straight into LDS: lane i's piece lands at lds_base + 16 * i
+// (global_load_lds_dwordx4; the LDS base travels in M0). Written in assembly because the compiler orders every later
+// LDS read behind such a load, whichever buffer it reads, which would undo the prefetch; so the compiler does not
+// count these loads either, and whoever reads the pieces waits for them (vmcnt) and for the other waves (barrier).
+__device__ __forceinline__ void copy_to_lds(const bf16* src, const bf16* lds_base) {
+  const unsigned base = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) bf16*)lds_base;
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+}
+// the same with the source as a scalar address (the same on all lanes) plus each lane's offset in bytes
+__device__ __forceinline__ void copy_to_lds(const bf16* src, unsigned lane_bytes, const bf16* lds_base) {
+  const unsigned base = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) bf16*)lds_base;
+  const uint64_t a = (uint64_t)src;       // into scalar registers, whatever the compiler made of the address so far
+  const uint64_t scalar = ((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(a >> 32)) << 32) |
+                          (unsigned)__builtin_amdgcn_readfirstlane((int)a);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_bytes), "s"(scalar), "s"(base) : "memory", "m0");
+}
+
+// the largest / the sum of a value over the four lanes that hold one column (they differ in lane bits 4 and 5),
+// by the row and half swaps of gfx950: no trip through LDS
+__device__ __forceinline__ float column_max(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float column_sum(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+template <bool PS16>
+__global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) void attention_tile_kernel(
+    const bf16* __restrict__ q, long q_ld, const bf16* __restrict__ plane, const int* __restrict__ block_tables,
+    int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ tiles,
+    bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
+    int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits, int min_steps,
+    int split_stride, int* __restrict__ row_splits) {
+  constexpr int NB = TNB;
+  __shared__ __attribute__((aligned(16))) bf16 k_lds[TBUF][TCH * 8];
+  __shared__ __attribute__((aligned(16))) bf16 v_lds[TBUF][TCH * 8];
+  const int page_size = PS16 ? 16 : page_size_arg;
+  const int tile = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  // the wave's number is the same on all its lanes: said so, what follows from it is scalar arithmetic and branches
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c16 = lane & 15, g = lane >> 4;
+  const int t_row0 = tiles[tile].x, t_rows = tiles[tile].y;
+  const int* bt = block_tables + (long)row_seq[t_row0] * bt_ld;
+  const int tp_first = positions[t_row0], tp_last = tp_first + t_rows - 1;
+
+  // the wave's rows of the tile; a wave past the tile's last row only helps with the copies
+  const int rows_per_wave = (16 * NB) / group_size;
+  const int n_rows = max(0, min(rows_per_wave, t_rows - wave * rows_per_wave));
+  const bool active = n_rows > 0;
+  const int row0 = t_row0 + (active ? wave * rows_per_wave : 0);
+  const int p_first = tp_first + (active ? wave * rows_per_wave : 0);
+  const int p_last = p_first + n_rows - 1;
+
+  int col_row[NB], col_head[NB], col_pos[NB], col_lo[NB];
+  bool col_ok[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int c = nb * 16 + c16;
+    const int ro = c / group_size;
+    col_ok[nb] = ro < n_rows;
+    col_row[nb] = row0 + (col_ok[nb] ? ro : 0);
+    col_head[nb] = kvh * group_size + c % group_size;
+    col_pos[nb] = col_ok[nb] ? p_first + ro : -1;
+    col_lo[nb] = (window > 0 && col_pos[nb] - window + 1 > 0) ? col_pos[nb] - window + 1 : 0;
+  }
+  bf16x8 qb[NB][DC];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) {
+      const int d = dc * 32 + g * 8;
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (col_ok[nb] && d < HD) v = load8(q + (long)col_row[nb] * q_ld + (long)col_head[nb] * HD + d);
+      qb[nb][dc] = v;
+    }
+
+  // the tile's keys and this workgroup's share of them, as in the wave kernel
+  const int t_lo = (window > 0 && tp_first - window + 1 > 0) ? tp_first - window + 1 : 0;   // first key any row sees
+  const int k_lo = t_lo & ~31;
+  const int k_hi = tp_last + 1;
+  const int n_steps = (k_hi - k_lo + 31) / 32;
+  int item_splits = n_splits;
+  if (min_steps > 0) item_splits = max(1, min(n_splits, n_steps / min_steps));
+  if (split >= item_splits) return;                   // the whole workgroup, before any barrier
+  if (row_splits && kvh == 0 && split == 0 && tid < t_rows) row_splits[t_row0 + tid] = item_splits;
+  const int per_split = (n_steps + item_splits - 1) / item_splits;
+  const int s_begin = split * per_split;
+  const int s_end = min(n_steps, s_begin + per_split);
+  const int w_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;    // first key the wave sees
+  const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+
+  const long page_stride = 2L * n_kv_heads * page_size * HD;
+  const long k_head = (long)kvh * page_size * HD;
+  const long v_head = ((long)n_kv_heads + kvh) * page_size * HD;
+
+  f32x4 o[NB][DB];
+  float m[NB], l[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    m[nb] = -INFINITY;
+    l[nb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) o[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  // Page ids: every wave keeps, in a line of LDS of its own, the pages of a run of 64 16-key tiles (32 steps),
+  // fetched by one vector load a run; a step reads its two from there. (Fetched step by step they would be scalar
+  // loads, and the waits for LDS data wait for outstanding scalar loads as well: a round trip to memory every step.)
+  __shared__ int run_pages[TW][64];
+  int run_first = s_begin;
+  auto load_run = [&](int s0) {
+    const int key0 = k_lo + (2 * s0 + lane) * 16;
+    run_pages[wave][lane] = bt[key0 < k_hi ? (PS16 ? key0 >> 4 : key0 / page_size) : 0];
+    run_first = s0;
+  };
+
+  // A lane's pieces of a step as offsets inside a page: they never change. With a head size in steps of 32 all
+  // pieces of a fetch lie in the same 16-key tile, and the page's address is scalar.
+  constexpr bool T_UNIFORM = HD % 32 == 0;
+  unsigned k_off[TPT], v_off[TPT];       // in elements; less than a page
+  int piece_t[TPT];
+#pragma unroll
+  for (int j = 0; j < TPT; ++j) {
+    const int c = tid + j * (TW * 64);                      // the piece's index in LDS
+    const int t = c / (2 * HD);                             // keys and values alike
+    piece_t[j] = T_UNIFORM ? __builtin_amdgcn_readfirstlane(t) : t;
+    k_off[j] = (unsigned)k_head + (c & 15) * HD + ((c >> 4) % NCH) * 8;
+    v_off[j] = (unsigned)v_head + (((c >> 5) % DB) * 16 + (c & 15)) * page_size + ((c >> 4) & 1) * 8;
+  }
+
+  // A step on its way from the pages to LDS buffer `buf`. A 16-key tile past the tile's keys reads page 0 (always
+  // mapped); its scores are masked below, and so are its values (see `values`).
+  auto stage = [&](int s, int buf) {
+    if (s - run_first >= 32) load_run(s);
+    long kbase[2], vbase[2];  // offsets from the plane, so that every load below is plainly one from global memory
+    const int2 pages = *reinterpret_cast<const int2*>(&run_pages[wave][2 * (s - run_first)]);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key0 = k_lo + s * 32 + t * 16;
+      const int pg = __builtin_amdgcn_readfirstlane(t ? pages.y : pages.x);
+      const long page = (long)(key0 < k_hi ? pg : 0) * page_stride;
+      const int slot0 = PS16 ? 0 : key0 % page_size;
+      kbase[t] = page + (long)slot0 * HD;
+      vbase[t] = page + slot0;
+    }
+#pragma unroll
+    for (int j = 0; j < TPT; ++j) {
+      if (TCH % (TW * 64) != 0 && wave * 64 + j * (TW * 64) >= TCH) break;
+      if (T_UNIFORM) copy_to_lds(plane + kbase[piece_t[j]], k_off[j] * 2, &k_lds[buf][(wave + j * TW) * 512]);
+      else copy_to_lds(plane + (kbase[piece_t[j]] + k_off[j]), &k_lds[buf][(wave + j * TW) * 512]);
+    }
+#pragma unroll
+    for (int j = 0; j < TPT; ++j) {
+      if (TCH % (TW * 64) != 0 && wave * 64 + j * (TW * 64) >= TCH) break;
+      if (T_UNIFORM) copy_to_lds(plane + vbase[piece_t[j]], v_off[j] * 2, &v_lds[buf][(wave + j * TW) * 512]);
+      else copy_to_lds(plane + (vbase[piece_t[j]] + v_off[j]), &v_lds[buf][(wave + j * TW) * 512]);
+    }
+  };
+  // the copies this wave has issued are in LDS
+  auto staged = [&]() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); };
+
+  // S^T of one step, one 16-key tile after the other (its keys are asked for together), dc by dc over the column
+  // blocks' independent sums
+  auto scores = [&](int buf, f32x4 (&st)[2][NB]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      bf16x8 ka[DC];
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) {
+        const int d = dc * 32 + g * 8;
+        const bool d_ok = (HD % 32 == 0) || d < HD;
+        ka[dc] = load8(&k_lds[buf][(((t * NCH + (d_ok ? dc * 4 + g : 0)) * 16) + c16) * 8]);
+        if (!d_ok) ka[dc] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) st[t][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          st[t][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[dc], qb[nb][dc], st[t][nb], 0, 0, 0);
+    }
+  };
+  // a step's scores without the keys that a column may not see; a step inside every column's range needs none of it
+  auto mask = [&](int s, f32x4 (&st)[2][NB]) {
+    const int kb = k_lo + s * 32;
+    const bool ok0 = kb < k_hi, ok1 = kb + 16 < k_hi;
+    if (ok0 && ok1 && kb + 31 <= p_first && kb >= lo_last) return;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + t * 16 + g * 4 + i;
+          const bool ok = (t ? ok1 : ok0) && key <= col_pos[nb] && key >= col_lo[nb];
+          st[t][nb][i] = ok ? st[t][nb][i] : -INFINITY;
+        }
+  };
+  // running maximum and sum per column, P in bfloat16 as the B operand of the second product
+  auto softmax = [&](const f32x4 (&st)[2][NB], bf16x8 (&pb)[NB], float (&alpha)[NB]) -> bool {
+    bool grew = false;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float sc[8];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float v = st[t][nb][i];
+          sc[t * 4 + i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+      tmax = column_max(tmax) * scale_log2;
+      // the exponent follows the running maximum in jumps, as in the wave kernel
+      const bool move = tmax > m[nb] + 8.f || m[nb] == -INFINITY;
+      const float m_new = move ? fmaxf(m[nb], tmax) : m[nb];
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      grew = grew || (move && m_new > m[nb]);
+      alpha[nb] = __builtin_amdgcn_exp2f(m[nb] - m_use);
+      float psum = 0.f;
+      bf16x8 pv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(sc[e], scale_log2, -m_use));
+        psum += p;
+        pv[e] = static_cast<__bf16>(p);
+      }
+      pb[nb] = pv;
+      l[nb] = l[nb] * alpha[nb] + psum;
+      m[nb] = m_new;
+    }
+    return __builtin_amdgcn_ballot_w64(grew) != 0;
+  };
+  // O^T = O^T * alpha + V^T . P^T; while no column of the wave has a new maximum every alpha is exactly 1.
+  // EDGE: the step holds keys that no row of the tile may see (past its last position, before its first window,
+  // past its last page). Their weights are zero, but their values are whatever an earlier owner of the page left,
+  // possibly not even finite: they are replaced by zeros before the product.
+  auto values = [&](int s, int buf, const bf16x8 (&pb)[NB], const float (&alpha)[NB], bool rescale, const bool EDGE) {
+    if (rescale) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[nb][db][i] *= alpha[nb];
+    }
+    bool dead[8];
+    if (EDGE) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = k_lo + s * 32 + (e >> 2) * 16 + g * 4 + (e & 3);
+        dead[e] = !(key <= tp_last && key >= t_lo);
+      }
+    }
+    constexpr int HALF = (DB + 1) / 2;      // the head in two halves: as many operands in registers at a time
+#pragma unroll
+    for (int h = 0; h < DB; h += HALF) {
+      bf16x8 va[HALF];
+#pragma unroll
+      for (int db = h; db < h + HALF && db < DB; ++db) {
+        const bf16* vp = &v_lds[buf][((db * 2 + (g >> 1)) * 16 + c16) * 8 + (g & 1) * 4];
+        const bf16x4 h0 = load4(vp), h1 = load4(vp + DB * 256);
+        va[db - h] = (bf16x8){h0[0], h0[1], h0[2], h0[3], h1[0], h1[1], h1[2], h1[3]};
+        if (EDGE) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (dead[e]) va[db - h][e] = static_cast<__bf16>(0.f);
+        }
+      }
+#pragma unroll
+      for (int db = h; db < h + HALF && db < DB; ++db)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[db - h], pb[nb], o[nb][db], 0, 0, 0);
+    }
+  };
+  // inside: every key of step s is one that some row of the tile sees
+  auto inside = [&](int s) { return k_lo + s * 32 + 31 <= tp_last && k_lo + s * 32 >= t_lo; };
+  // a wave skips the steps whose keys all lie past its last row or before its first window
+  auto mine = [&](int s) { return active && s < s_end && k_lo + s * 32 <= p_last && k_lo + s * 32 + 31 >= w_lo; };
+
+  if (s_begin < s_end) {
+    // Steps s_begin and s_begin + 1 go to LDS before the loop; the loop's turn s copies step s + 2, multiplies out
+    // the scores of step s + 1 and finishes step s. Buffer of step s: (s - s_begin) % TBUF.
+    load_run(s_begin);
+    stage(s_begin, 0);
+    if (s_begin + 1 < s_end) stage(s_begin + 1, 1);
+    staged();
+    __syncthreads();
+    f32x4 st_cur[2][NB], st_next[2][NB];
+    if (mine(s_begin)) {
+      scores(0, st_cur);
+      mask(s_begin, st_cur);
+    }
+    int buf = 0;                                   // of step s
+    for (int s = s_begin; s < s_end; ++s) {
+      const int buf1 = buf + 1 == TBUF ? 0 : buf + 1, buf2 = buf1 + 1 == TBUF ? 0 : buf1 + 1;
+      if (s + 2 < s_end) stage(s + 2, buf2);
+      const bool cur = mine(s), next = mine(s + 1);
+      bf16x8 pb[NB];
+      float alpha[NB];
+      if (next) scores(buf1, st_next);
+      if (cur) {
+        const bool rescale = softmax(st_cur, pb, alpha);
+        values(s, buf, pb, alpha, rescale, !inside(s));
+      }
+      if (next) mask(s + 1, st_next);
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) st_cur[t][nb] = st_next[t][nb];
+      buf = buf1;
+      // everyone has read step s's buffer (the copy of step s + 3 overwrites it) and step s + 2 has arrived
+      staged();
+      __syncthreads();
+    }
+  }
+
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const float lt = column_sum(l[nb]);
+    if (!col_ok[nb]) continue;
+    if (item_splits == 1) {
+      const float inv = 1.f / lt;
+      bf16* dst = out + (long)col_row[nb] * out_ld + (long)col_head[nb] * HD + g * 4;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        bf16x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = static_cast<__bf16>(o[nb][db][i] * inv);
+        *reinterpret_cast<bf16x4*>(dst + db * 16) = w;
+      }
+    } else {
+      const long slot = ((long)col_row[nb] * n_heads + col_head[nb]) * split_stride + split;
       float* dst = part_o + slot * HD + g * 4;
 #pragma unroll
       for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + db * 16) = o[nb][db];
@@ -448,58 +821,91 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_rows_kernel(const flo
 }
 
 TIS_EXPORT int tis_attention_mfma_head_dim() { return HD; }
+// columns (row, query head of a group) that one wave of a tile holds; a tile has four waves
+TIS_EXPORT int tis_attention_mfma_tile_columns() { return 16 * TNB; }
 
 // items: (first row, rows) pairs; the rows of an item are consecutive positions of one request and
-// rows * group_size <= 16 * nb. Null: n_items single rows, item i being row i. part_o / part_ml: workspace for
-// n_splits > 1, [rows][heads][splits][HD] floats and [rows][heads][splits] float pairs. min_steps > 0: an item
-// uses min(n_splits, its steps of 32 keys / min_steps) splits, and row_splits [rows] receives each row's count.
+// rows * group_size <= 16 * nb. Null: n_items single rows, item i being row i. tiles: (first row, rows) pairs for the
+// workgroup kernel, rows <= 4 * (tis_attention_mfma_tile_columns() / group_size); items and tiles together hold every row once.
+// n_splits / tile_splits: what the grid offers an item / a tile. part_o / part_ml: workspace where either exceeds
+// one, [rows][heads][S][HD] floats and [rows][heads][S] float pairs, S the larger of the two. min_steps > 0 (tiles:
+// tile_min_steps): an item uses min(n_splits, its steps of 32 keys / min_steps) splits, and row_splits [rows]
+// receives each row's count.
 TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
                                   const int* row_seq, const int* positions, const int* items, int n_items, int nb,
-                                  void* out, long out_ld, float* part_o, float* part_ml, int rows, int n_heads,
-                                  int n_kv_heads, int head_dim, int page_size, int window, float scale, int n_splits,
-                                  int min_steps, int* row_splits, hipStream_t stream) {
-  if (n_items == 0 || rows == 0) return 0;
+                                  const int* tiles, int n_tiles, void* out, long out_ld, float* part_o,
+                                  float* part_ml, int rows, int n_heads, int n_kv_heads, int head_dim, int page_size,
+                                  int window, float scale, int n_splits, int min_steps, int tile_splits,
+                                  int tile_min_steps, int* row_splits, hipStream_t stream) {
+  if ((n_items == 0 && n_tiles == 0) || rows == 0) return 0;
+  if (n_items < 0 || n_tiles < 0 || (n_tiles > 0 && !tiles)) return tis_fail("attention_mfma: bad item counts %d, %d", n_items, n_tiles);
   if (head_dim != HD) return tis_fail("attention_mfma: built for head size %d, called with %d", HD, head_dim);
   if (n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads)
     return tis_fail("attention_mfma: %d query heads over %d key/value heads", n_heads, n_kv_heads);
   const int group = n_heads / n_kv_heads;
-  if (nb != 1 && nb != 2 && nb != 4) return tis_fail("attention_mfma: %d column blocks; 1, 2 or 4 are built", nb);
-  if (group > 16 * nb) return tis_fail("attention_mfma: a group of %d query heads does not fit %d columns", group, 16 * nb);
+  if (n_items > 0) {
+    if (nb != 1 && nb != 2 && nb != 4) return tis_fail("attention_mfma: %d column blocks; 1, 2 or 4 are built", nb);
+    if (group > 16 * nb) return tis_fail("attention_mfma: a group of %d query heads does not fit %d columns", group, 16 * nb);
+  } else {
+    n_splits = 1;
+  }
+  if (n_tiles > 0 && group > 16 * TNB) return tis_fail("attention_mfma: a group of %d query heads does not fit a tile's wave", group);
+  if (n_tiles == 0) tile_splits = 1;
   if (page_size < 16 || page_size % 16) return tis_fail("attention_mfma: page size %d is no multiple of 16", page_size);
-  if (n_splits < 1 || n_splits > 65535 || n_kv_heads > 65535) return tis_fail("attention_mfma: bad grid %d x %d", n_kv_heads, n_splits);
-  if (n_splits > 1 && (!part_o || !part_ml)) return tis_fail("attention_mfma: %d splits need a workspace", n_splits);
+  if (n_splits < 1 || n_splits > 65535 || tile_splits < 1 || tile_splits > 65535 || n_kv_heads > 65535)
+    return tis_fail("attention_mfma: bad grid %d x %d (tiles: %d)", n_kv_heads, n_splits, tile_splits);
+  const int stride = n_splits > tile_splits ? n_splits : tile_splits;
+  if (stride > 1 && (!part_o || !part_ml)) return tis_fail("attention_mfma: %d splits need a workspace", stride);
   if (min_steps < 0 || (min_steps > 0 && n_splits > 1 && !row_splits))
     return tis_fail("attention_mfma: splits chosen item by item (min_steps=%d) need the per-row count array", min_steps);
-  if (min_steps == 0 || n_splits == 1) row_splits = nullptr;
+  if (n_tiles > 0 && stride > 1 && (tile_min_steps < 1 || !row_splits || (n_items > 0 && min_steps < 1)))
+    return tis_fail("attention_mfma: tiles beside split key ranges need the per-row count array and a minimum of steps");
+  if (stride == 1 || (n_tiles == 0 && min_steps == 0)) row_splits = nullptr;
   if ((q_ld % 8) || (out_ld % 4) || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)plane % 16))
     return tis_fail("attention_mfma: q, out and the cache plane must be 16-byte aligned with row strides in steps of 8");
-  dim3 grid(n_items, n_kv_heads, n_splits);
   const float scale_log2 = scale * 1.4426950408889634f;
+  int rc = 0;
+  if (n_items > 0) {
+    dim3 grid(n_items, n_kv_heads, n_splits);
 #define LAUNCH(NBV, PSV)                                                                                              \
   attention_mfma_kernel<NBV, PSV><<<grid, 64, 0, stream>>>(                                                      \
       (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)items,     \
       (bf16*)out, out_ld, part_o, (float2*)part_ml, group, n_kv_heads, n_heads, page_size, window, scale_log2,   \
-      n_splits, min_steps, row_splits)
-  if (page_size == 16) {
-    if (nb == 1) LAUNCH(1, true);
-    else if (nb == 2) LAUNCH(2, true);
-    else LAUNCH(4, true);
-  } else {
-    if (nb == 1) LAUNCH(1, false);
-    else if (nb == 2) LAUNCH(2, false);
-    else LAUNCH(4, false);
-  }
+      n_splits, min_steps, stride, row_splits)
+    if (page_size == 16) {
+      if (nb == 1) LAUNCH(1, true);
+      else if (nb == 2) LAUNCH(2, true);
+      else LAUNCH(4, true);
+    } else {
+      if (nb == 1) LAUNCH(1, false);
+      else if (nb == 2) LAUNCH(2, false);
+      else LAUNCH(4, false);
+    }
 #undef LAUNCH
-  int rc = tis_launch_status("attention_mfma");
-  if (rc) return rc;
-  if (n_splits > 1) {
+    rc = tis_launch_status("attention_mfma");
+    if (rc) return rc;
+  }
+  if (n_tiles > 0) {
+    dim3 grid(n_tiles, n_kv_heads, tile_splits);
+#define LAUNCH(PSV)                                                                                                   \
+  attention_tile_kernel<PSV><<<grid, TW * 64, 0, stream>>>(                                                      \
+      (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)tiles,     \
+      (bf16*)out, out_ld, part_o, (float2*)part_ml, group, n_kv_heads, n_heads, page_size, window, scale_log2,   \
+      tile_splits, tile_min_steps, stride, row_splits)
+    if (page_size == 16) LAUNCH(true);
+    else LAUNCH(false);
+#undef LAUNCH
+    rc = tis_launch_status("attention_tile");
+    if (rc) return rc;
+  }
+  if (stride > 1) {
     if ((long)rows * n_heads > 8192) {
       attention_merge_rows_kernel<<<rows, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld,
-                                                                n_heads, n_splits, row_splits);
+                                                                n_heads, stride, row_splits);
     } else {
       dim3 mgrid(rows, n_heads);
       attention_merge_kernel<<<mgrid, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld,
-                                                            n_heads, n_splits, row_splits);
+                                                            n_heads, stride, row_splits);
     }
     rc = tis_launch_status("attention_merge");
   }

@@ -84,8 +84,8 @@ _SIGNATURES["gemm_library"] = ("tis_gemm_library", {
     "tis_gemm_library": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _I, _P],
 })
 _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
-    "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I,
-                           _P, _P],
+    "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F,
+                           _I, _I, _I, _I, _P, _P],
 })
 
 _libs = {}
@@ -108,42 +108,74 @@ _ATTN_PROMPT_TARGET_WAVES = 2048  # what the grid offers where rows of prompts a
 _ATTN_PROMPT_SPLIT_MAX_ROWS = 512 # ... and the batch is small; a long portion fills the chip by its rows alone
 _ATTN_PROMPT_MIN_STEPS = 8         # steps of 32 keys below which a prompt item's split is not worth its merge
 _ATTN_MIN_SPLIT_KEYS = 128      # a split shorter than this costs more in merging than it gains in spreading
+_ATTN_TILE_WAVES = 4            # waves of the workgroup that takes a tile of a long portion
+_ATTN_TILE_GROUPS = 512         # workgroups of the tile kernel that the chip runs side by side
+_ATTN_TILE_MIN_STEPS = 8        # steps of 32 keys below which a tile's split is not worth its merge
+_ATTN_TILE_SPLIT_SLACK = 1.5    # a split may be this much longer than an even share of all steps
+_ATTN_TILE_MIN_WORK = 4000      # tile steps times key/value heads below which the one-wave kernel is the faster
 _ATTN_WORKSPACE_FLOATS = 16 << 20
 
 
-def attention_items(seq_rows, group_size: int):
-    """Work items of the matrix-core attention kernel for the rows of one stage.
+def tile_columns(head_dim: int) -> int:
+    """Columns (row, query head of a group) of one wave of the tile kernel, as the kernel source sets them."""
+    return 32 if head_dim <= 128 else 16
 
-    seq_rows: (first row, first position, rows) per request. Returns (column blocks per item, int32 array of
-    (first row, rows) lines):
-    an item holds consecutive rows of one request, rows * group_size <= 16 * blocks. When no request has more
-    than one row the list is simply every row in order, which the kernel knows without being given a list.
+
+def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: int = 0):
+    """Work items of the matrix-core attention kernels for the rows of one stage.
+
+    seq_rows: (first row, first position, rows) per request. Returns (column blocks per item, items, tiles, steps):
+    items and tiles are int32 arrays of (first row, rows) lines that together hold every row once, steps is the
+    number of 32-key steps that all tiles walk together (the kernel's work, by which its key splits are sized).
+    An item (one wave) holds consecutive rows of one request, rows * group_size <= 16 * blocks. When no request has
+    more than one row the list is simply every row in order, which the kernel knows without being given a list.
+    A tile (a workgroup of four waves, `tile_cols` columns each; 0: no tiles) takes up to 4 * (tile_cols // group_size)
+    consecutive rows of a portion that fills at least half of one. Tiles are made only where their steps times
+    `n_kv_heads` (the workgroups' work) reach _ATTN_TILE_MIN_WORK (0: always): a tile's waves walk its keys in
+    lockstep, which pays when there is work for every compute unit and costs on a short prompt.
     """
+    none = np.zeros((0, 2), dtype=np.int32)
     single = all(n <= 1 for _, _, n in seq_rows)
-    nb = 1 if single else 2
-    # 64-column items halve what a prompt reads of its keys and values; they pay (some 10 % at 8,192 rows) once
-    # there are enough of them to fill the chip, and cost where a few long chains of steps set the time
-    if not single and group_size <= 64 and sum(-(-n // max(1, 64 // group_size)) for _, _, n in seq_rows) >= 384:
+    if single:
+        nb = 1
+        while group_size > 16 * nb:
+            nb *= 2
+        return nb, np.asarray([(first, 1) for first, _, n in seq_rows if n], dtype=np.int32).reshape(-1, 2), none, 0
+    tile_rows = _ATTN_TILE_WAVES * (tile_cols // group_size)
+    tiled = [(f, p0, n) for f, p0, n in seq_rows if tile_rows and n >= max(2, tile_rows // 2)]
+    if tiled and n_kv_heads:
+        work = sum(int(((p0 + np.minimum(np.arange(0, n, tile_rows) + tile_rows, n) + 31) // 32).sum())
+                   for _, p0, n in tiled) * n_kv_heads
+        if work < _ATTN_TILE_MIN_WORK:
+            tiled = []
+    taken = {f for f, _, _ in tiled}
+    rest = [(f, p0, n) for f, p0, n in seq_rows if n > 0 and f not in taken]
+
+    def cut(segments, per_item):
+        if not segments:
+            return none, 0
+        firsts, counts, keys = [], [], []
+        for first, p0, n in segments:
+            r = np.arange(0, n, per_item, dtype=np.int64)
+            cnt = np.minimum(per_item, n - r)
+            firsts.append(first + r)
+            counts.append(cnt)
+            keys.append(p0 + r + cnt)
+        firsts, counts, keys = np.concatenate(firsts), np.concatenate(counts), np.concatenate(keys)
+        # those with the most keys first: under a causal mask the last rows of a prompt are the longest, and
+        # started last they would run on alone while the rest of the chip idles
+        order = np.argsort(-keys, kind="stable")
+        return np.stack((firsts[order], counts[order]), axis=1).astype(np.int32), int(((keys + 31) // 32).sum())
+
+    nb = 2
+    # 64-column items halve what a portion reads of its keys and values; they pay once there are enough of them
+    # to fill the chip, and cost where a few long chains of steps set the time
+    if group_size <= 64 and sum(-(-n // max(1, 64 // group_size)) for _, _, n in rest) >= 384:
         nb = 4
     while group_size > 16 * nb:
         nb *= 2
-    per_item = max(1, (16 * nb) // group_size)
-    if single:
-        return nb, np.asarray([(first, 1) for first, _, n in seq_rows if n], dtype=np.int32).reshape(-1, 2)
-    firsts, counts, keys = [], [], []
-    for first, p0, n in seq_rows:
-        if n <= 0:
-            continue
-        r = np.arange(0, n, per_item, dtype=np.int64)
-        cnt = np.minimum(per_item, n - r)
-        firsts.append(first + r)
-        counts.append(cnt)
-        keys.append(p0 + r + cnt)
-    firsts, counts, keys = np.concatenate(firsts), np.concatenate(counts), np.concatenate(keys)
-    # the items with the most keys first: under a causal mask the last rows of a prompt are the longest, and
-    # started last they would run on alone while the rest of the chip idles
-    order = np.argsort(-keys, kind="stable")
-    return nb, np.stack((firsts[order], counts[order]), axis=1).astype(np.int32)
+    tiles, steps = cut(tiled, tile_rows)
+    return nb, cut(rest, max(1, (16 * nb) // group_size))[0], tiles, steps
 
 
 def _rows_view(t: torch.Tensor, what: str):
@@ -188,16 +220,18 @@ class HipOps:
     # ---- planning on the host --------------------------------------------------------------------------
     def register_attention(self, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
         """An attention mixer announces its shape, so that each step's work items are planned once, up front."""
-        self._attn_groups.add(n_heads // n_kv_heads)
+        self._attn_groups.add((n_heads // n_kv_heads, tile_columns(head_dim), n_kv_heads))
 
     def plan_rows(self, seq_rows, add):
         """Called while a step's arrays are packed: returns {name: (packed array id, host values...)}."""
         plans = {}
         if self.dtype == torch.bfloat16:
-            for group in sorted(self._attn_groups):
-                nb, items = attention_items(seq_rows, group)
-                if nb <= 4 and len(items):
-                    plans[("attention_items", group)] = (add(items), len(items), nb)
+            for group, cols, kvh in sorted(self._attn_groups):
+                nb, items, tiles, steps = attention_items(seq_rows, group, cols, kvh)
+                if nb <= 4 and (len(items) or len(tiles)):
+                    # one array: the items' lines, then the tiles'
+                    plans[("attention_items", group, cols, kvh)] = (add(np.concatenate((items, tiles))), len(items),
+                                                                    nb, len(tiles), steps)
         return plans
 
     # ---- helpers -------------------------------------------------------------------------------------
@@ -515,45 +549,63 @@ class HipOps:
         group = n_heads // n_kv_heads
         if (self.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 16 == 0
                 and group <= 64 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0):
-            plan = batch.extras.get(("attention_items", group))
-            if plan is None:        # a caller that did not plan (a kernel test): plan now
-                nb, host_items = attention_items(batch.seq_rows, group)
-                items = torch.from_numpy(np.ascontiguousarray(host_items)).reshape(-1).to(self.device)
-                plan = (items, len(host_items), nb)
-            items, n_items, nb = plan
+            cols = tile_columns(head_dim)
+            plan = batch.extras.get(("attention_items", group, cols, n_kv_heads))
+            if plan is None:        # a caller that did not plan (a kernel test): plan now, tiles wherever they fit
+                nb, host_items, host_tiles, steps = attention_items(batch.seq_rows, group, cols)
+                both = np.ascontiguousarray(np.concatenate((host_items, host_tiles)))
+                plan = (torch.from_numpy(both).reshape(-1).to(self.device), len(host_items), nb, len(host_tiles), steps)
+            lines, n_items, nb, n_tiles, tile_steps = plan
+            lines = lines.reshape(-1)
+            items = lines[:2 * n_items] if n_items else None
+            tiles = lines[2 * n_items:] if n_tiles else None
             if batch.max_seq_rows <= 1 and n_items == n:
                 items = None        # single rows in order: the kernel needs no list
             lib = self._attn_mfma.get(head_dim)
             if lib is None:
                 lib = self._attn_mfma[head_dim] = library(f"attention_mfma@{head_dim}")
-            single = items is None
-            # decoded tokens: every request's keys are cut into the same number of splits, enough to spread a short
-            # batch over the chip. Prompt rows: the grid offers more splits than the chip needs and every item takes
-            # as many as its own length deserves (the kernel decides, from _ATTN_PROMPT_MIN_STEPS), because the last
-            # rows of a long prompt would otherwise run on alone long after the first have finished.
-            target = _ATTN_PROMPT_TARGET_WAVES if (not single and n <= _ATTN_PROMPT_SPLIT_MAX_ROWS) else _ATTN_TARGET_WAVES
-            # a lone request or two: shorter splits still pay, because so few waves would leave most of the chip idle
-            min_keys = _ATTN_MIN_SPLIT_KEYS // 2 if n_items * n_kv_heads <= 8 else _ATTN_MIN_SPLIT_KEYS
-            n_splits = max(1, min(-(-target // (n_items * n_kv_heads)), batch.max_kv_len // min_keys))
-            min_steps = 0 if single else _ATTN_PROMPT_MIN_STEPS
+                built = lib.cdll.tis_attention_mfma_tile_columns()
+                if built != cols:
+                    raise KernelError(f"attention: the kernel's tiles hold {built} columns a wave, the planner "
+                                      f"assumes {cols}")
+            single = items is None and n_tiles == 0
+            n_splits, min_steps, tile_splits, tile_min_steps = 1, 0, 1, _ATTN_TILE_MIN_STEPS
+            if n_items:
+                # decoded tokens: every request's keys are cut into the same number of splits, enough to spread a
+                # short batch over the chip. Prompt rows: the grid offers more splits than the chip needs and every
+                # item takes as many as its own length deserves (the kernel decides, from _ATTN_PROMPT_MIN_STEPS),
+                # because the last rows of a long prompt would otherwise run on alone long after the first have finished.
+                target = _ATTN_PROMPT_TARGET_WAVES if (not single and n <= _ATTN_PROMPT_SPLIT_MAX_ROWS) else _ATTN_TARGET_WAVES
+                # a lone request or two: shorter splits still pay, because so few waves would leave most of the chip idle
+                min_keys = _ATTN_MIN_SPLIT_KEYS // 2 if n_items * n_kv_heads <= 8 else _ATTN_MIN_SPLIT_KEYS
+                n_splits = max(1, min(-(-target // (n_items * n_kv_heads)), batch.max_kv_len // min_keys))
+                min_steps = 0 if single else _ATTN_PROMPT_MIN_STEPS
+            if n_tiles:
+                # a tile's keys are cut where it alone would run longer than an even share of all tiles' steps
+                # (the last rows of a long prompt); a split is never shorter than _ATTN_TILE_MIN_STEPS
+                share = tile_steps * n_kv_heads / _ATTN_TILE_GROUPS
+                tile_min_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
+                tile_splits = max(1, -(-batch.max_kv_len // 32) // tile_min_steps)
             # partial results of split key ranges live in one workspace of fixed size, allocated once and never
             # moved (captured graphs hold its address); fewer splits where it would not suffice
-            n_splits = max(1, min(n_splits, (_ATTN_WORKSPACE_FLOATS - n) // (n * n_heads * (head_dim + 2))))
+            most = max(1, (_ATTN_WORKSPACE_FLOATS - n) // (n * n_heads * (head_dim + 2)))
+            n_splits, tile_splits = min(n_splits, most), min(tile_splits, most)
+            stride = max(n_splits, tile_splits)
             part_o = part_ml = row_splits = None
-            if n_splits > 1:
+            if stride > 1:
                 if self._workspace is None:
                     if torch.cuda.is_current_stream_capturing():
                         raise KernelError("the attention workspace must exist before a graph is captured")
                     self._workspace = torch.empty(_ATTN_WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
                 part_o = self._workspace
-                part_ml = self._workspace[n * n_heads * n_splits * head_dim:]
-                if min_steps:
-                    row_splits = self._workspace[n * n_heads * n_splits * (head_dim + 2):]
+                part_ml = self._workspace[n * n_heads * stride * head_dim:]
+                if not single:
+                    row_splits = self._workspace[n * n_heads * stride * (head_dim + 2):]
             lib.tis_attention_mfma(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0),
-                                   _ptr(batch.row_seq), _ptr(batch.positions), _ptr(items), n_items, nb, _ptr(out),
-                                   out.stride(0), _ptr(part_o), _ptr(part_ml), n, n_heads, n_kv_heads, head_dim,
-                                   page_size, int(window), float(scale), n_splits, min_steps, _ptr(row_splits),
-                                   self._stream())
+                                   _ptr(batch.row_seq), _ptr(batch.positions), _ptr(items), n_items, nb, _ptr(tiles),
+                                   n_tiles, _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), n, n_heads,
+                                   n_kv_heads, head_dim, page_size, int(window), float(scale), n_splits, min_steps,
+                                   tile_splits, tile_min_steps, _ptr(row_splits), self._stream())
             return out
         self.attn_generic.tis_attention_generic(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),

@@ -49,7 +49,7 @@ def parse_segments(text: str):
 
 
 def attention_case(ops, a):
-    from .hip_ops import attention_items
+    from .hip_ops import attention_items, tile_columns
     nh, kvh, hd, ps = a.heads, a.kv_heads, a.head_dim, a.page_size
     segs = parse_segments(a.segments)
     pages = [-(-(p0 + n) // ps) for p0, n in segs]
@@ -68,9 +68,12 @@ def attention_case(ops, a):
                             row_seq=torch.tensor(row_seq, dtype=torch.int32, device=ops.device),
                             block_tables={"g": tables.to(ops.device)}, max_kv_len=max(p0 + n for p0, n in segs),
                             extras={}, n_rows=rows, max_seq_rows=max(n for _, n in segs), seq_rows=seq_rows)
-    nb, items = attention_items(seq_rows, nh // kvh)
-    batch.extras[("attention_items", nh // kvh)] = (torch.as_tensor(items, dtype=torch.int32).reshape(-1).to(ops.device),
-                                                    len(items), nb)
+    # --no-tiles: what the one-wave kernel alone makes of the same rows; --tiles: tiles however little work there is
+    nb, items, tiles, steps = attention_items(seq_rows, nh // kvh, 0 if a.no_tiles else tile_columns(hd),
+                                              0 if a.tiles else kvh)
+    import numpy as np
+    both = torch.from_numpy(np.ascontiguousarray(np.concatenate((items, tiles)))).reshape(-1).to(ops.device)
+    batch.extras[("attention_items", nh // kvh, tile_columns(hd), kvh)] = (both, len(items), nb, len(tiles), steps)
     us = graph_time(lambda: ops.paged_attention(q, plane, batch, "g", nh, kvh, hd), a.reps)
     kv_bytes = sum(p0 + n for p0, n in segs) * kvh * hd * 2 * 2
     flops = sum(4 * nh * hd * (n * p0 + n * (n + 1) / 2) for p0, n in segs)
@@ -102,6 +105,8 @@ def main(argv=None) -> int:
     at.add_argument("--kv-heads", type=int, default=3)
     at.add_argument("--head-dim", type=int, default=128)
     at.add_argument("--page-size", type=int, default=16)
+    at.add_argument("--no-tiles", action="store_true", help="long portions too go to the one-wave kernel")
+    at.add_argument("--tiles", action="store_true", help="long portions go to the workgroup kernel however few they are")
     pr = sub.add_parser("product")
     pr.add_argument("--rows", type=int, default=8)
     pr.add_argument("--out", type=int, default=8192)

@@ -123,6 +123,34 @@ def test_all_schedules_agree_with_each_other(backend):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", ["B", "C", "D"])
+def test_schedules_with_portions_on_the_tile_kernel(name, monkeypatch):
+    """The tiny models' prompts are too little work for the workgroup attention kernel to be chosen; here it is made
+    to take every portion that fills half a tile, and whole prompts, portions and mixed batches (with pages handed
+    out again) are compared with the plain implementation as elsewhere."""
+    from tiny_inference_server_amd.ops import hip_ops
+    monkeypatch.setattr(hip_ops, "_ATTN_TILE_MIN_WORK", 0)
+    planned = {"tiles": 0}
+    plan = hip_ops.attention_items
+
+    def counting(*args, **kw):
+        out = plan(*args, **kw)
+        planned["tiles"] += len(out[2])
+        return out
+    monkeypatch.setattr(hip_ops, "attention_items", counting)
+    lengths = [97, 50, 64, 37, 90, 18, 70]
+    reqs = requests_for(name, lengths, seed=8)
+    mixed, peak = H.mixed_trace(reqs, max_live=4, seed=6)
+    for trace, max_tokens in ((H.whole_trace(reqs), 512), (H.portions_trace(reqs, seed=4), 512), (mixed, peak)):
+        folder, eng = make_engine(name, "bfloat16", "hip", max_tokens=max_tokens)
+        main, heads = H.run_trace(eng, trace)
+        assert planned["tiles"] > 0          # whole prompts always fill tiles; the short portions of C may not
+        H.compare_with_plain(folder, reqs, main, heads, TOL["bfloat16"] * scale_of(folder, reqs), eng.config.mtp_heads)
+        eng.cache.check()
+        assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.gpu
 def test_long_context_decoding_in_bfloat16():
     """A prompt of 500 tokens in uneven portions, then 120 tokens one by one through captured graphs: keys are cut
     into several splits, pages are crossed, and every logit still matches the plain model."""

@@ -42,6 +42,21 @@ static constexpr int DB = HD / 16;          // 16-wide blocks of the head for P.
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x4 load4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
 
+// the largest / the sum of a value over the four lanes that hold one column (they differ in lane bits 4 and 5),
+// by the row and half swaps of gfx950: no trip through LDS
+__device__ __forceinline__ float column_max(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float column_sum(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // PS16: pages of exactly 16 tokens. A 16-key tile is then a whole page, page indices are shifts, and a lane's
 // offsets inside a page never change: the loads of a step need no address arithmetic beyond the page's base.
 template <int NB, bool PS16>
@@ -222,9 +237,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
           sv[t * 4 + i] = v;
           tmax = fmaxf(tmax, v);
         }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      tmax *= scale_log2;
+      tmax = column_max(tmax) * scale_log2;
       // m is the exponent that P, the sum and the output are taken relative to. It follows the running maximum
       // only when that has grown by more than 2^8 beyond it, so it settles after a row's first keys and the
       // rescaling below becomes rare; until then P stays below 256, well inside bfloat16, and sum and output
@@ -300,9 +313,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
   // the lane holds, for its column, the outputs d = db*16 + g*4 + {0..3}
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
-    float lt = l[nb];
-    lt += __shfl_xor(lt, 16, 64);
-    lt += __shfl_xor(lt, 32, 64);
+    const float lt = column_sum(l[nb]);
     if (!col_ok[nb]) continue;
     if (item_splits == 1) {
       const float inv = 1.f / lt;
@@ -361,21 +372,6 @@ __device__ __forceinline__ void copy_to_lds(const bf16* src, unsigned lane_bytes
   const uint64_t scalar = ((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(a >> 32)) << 32) |
                           (unsigned)__builtin_amdgcn_readfirstlane((int)a);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_bytes), "s"(scalar), "s"(base) : "memory", "m0");
-}
-
-// the largest / the sum of a value over the four lanes that hold one column (they differ in lane bits 4 and 5),
-// by the row and half swaps of gfx950: no trip through LDS
-__device__ __forceinline__ float column_max(float v) {
-  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
-  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
-}
-__device__ __forceinline__ float column_sum(float v) {
-  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
-  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 template <bool PS16>

@@ -765,9 +765,10 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_kernel(const float* _
   }
 }
 
-// The same merge for many rows (prompt portions): one workgroup a row, its four waves take the heads in turn, and a
-// row that was not split costs one load. With a workgroup per (row, head) the thousands of rows of a prompt would
-// mean tens of thousands of workgroups that each live for three round trips to memory.
+// The same merge for many rows (prompt portions): a workgroup takes four heads of a row, one a wave, and a row that
+// was not split costs one load. With a workgroup per (row, head) the thousands of rows of a prompt would mean tens of
+// thousands of workgroups; with a wave taking several heads in turn, each head's two round trips to memory follow
+// the previous head's.
 __global__ __launch_bounds__(MG * 64) void attention_merge_rows_kernel(const float* __restrict__ part_o,
                                                                        const float2* __restrict__ part_ml,
                                                                        bf16* __restrict__ out, long out_ld,
@@ -777,42 +778,42 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_rows_kernel(const flo
   const int n_splits = row_splits ? row_splits[row] : max_splits;
   if (n_splits <= 1) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int head = wave; head < n_heads; head += MG) {
-    const long base = (row * n_heads + head) * max_splits;
-    float acc[MD];
+  const int head = blockIdx.y * MG + wave;
+  if (head >= n_heads) return;
+  const long base = (row * n_heads + head) * max_splits;
+  float acc[MD];
 #pragma unroll
-    for (int j = 0; j < MD; ++j) acc[j] = 0.f;
-    float M = -INFINITY, L = 0.f;
-    for (int s0 = 0; s0 < n_splits; s0 += 64)
-      if (s0 + lane < n_splits) M = fmaxf(M, part_ml[base + s0 + lane].x);
+  for (int j = 0; j < MD; ++j) acc[j] = 0.f;
+  float M = -INFINITY, L = 0.f;
+  for (int s0 = 0; s0 < n_splits; s0 += 64)
+    if (s0 + lane < n_splits) M = fmaxf(M, part_ml[base + s0 + lane].x);
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
-    for (int s0 = 0; s0 < n_splits; s0 += 64) {
-      float w = 0.f;
-      if (s0 + lane < n_splits) {
-        const float2 ml = part_ml[base + s0 + lane];
-        if (ml.x != -INFINITY) {
-          w = exp2f(ml.x - M);
-          L += w * ml.y;
-        }
-      }
-      const int cnt = min(64, n_splits - s0);
-      for (int i = 0; i < cnt; ++i) {
-        const float wi = __shfl(w, i, 64);
-#pragma unroll
-        for (int j = 0; j < MD; ++j) {
-          const int d = j * 64 + lane;
-          if (d < HD && wi != 0.f) acc[j] += wi * part_o[(base + s0 + i) * HD + d];
-        }
+  for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+  for (int s0 = 0; s0 < n_splits; s0 += 64) {
+    float w = 0.f;
+    if (s0 + lane < n_splits) {
+      const float2 ml = part_ml[base + s0 + lane];
+      if (ml.x != -INFINITY) {
+        w = exp2f(ml.x - M);
+        L += w * ml.y;
       }
     }
+    const int cnt = min(64, n_splits - s0);
+    for (int i = 0; i < cnt; ++i) {
+      const float wi = __shfl(w, i, 64);
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
-#pragma unroll
-    for (int j = 0; j < MD; ++j) {
-      const int d = j * 64 + lane;
-      if (d < HD) out[row * out_ld + (long)head * HD + d] = static_cast<__bf16>(acc[j] / L);
+      for (int j = 0; j < MD; ++j) {
+        const int d = j * 64 + lane;
+        if (d < HD && wi != 0.f) acc[j] += wi * part_o[(base + s0 + i) * HD + d];
+      }
     }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+#pragma unroll
+  for (int j = 0; j < MD; ++j) {
+    const int d = j * 64 + lane;
+    if (d < HD) out[row * out_ld + (long)head * HD + d] = static_cast<__bf16>(acc[j] / L);
   }
 }
 
@@ -896,8 +897,9 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
   }
   if (stride > 1) {
     if ((long)rows * n_heads > 8192) {
-      attention_merge_rows_kernel<<<rows, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld,
-                                                                n_heads, stride, row_splits);
+      dim3 mgrid(rows, (n_heads + MG - 1) / MG);
+      attention_merge_rows_kernel<<<mgrid, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld,
+                                                                 n_heads, stride, row_splits);
     } else {
       dim3 mgrid(rows, n_heads);
       attention_merge_kernel<<<mgrid, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld,

@@ -5,15 +5,11 @@
 // choosing an algorithm for a shape takes as long as launching it, and the framework's path asks again on every
 // call (18 us a product measured on MI355X's host; a prompt step of 32 blocks issues 128 of them). Here the
 // descriptors and the algorithm of a shape are made once and kept, which leaves the launch itself (9.5 us).
-// Which of its kernels runs: the library's heuristic names several candidates; the first serves until the candidates
-// have been timed, each a few times on a call's own operands (into a scratch result), and then the fastest does.
-// (The heuristic's first choice for the q/k/v projection of a 2,048-token step is 15 % behind its second on MI355X.)
+// The kernels that run, and so the results, are the library's own choice for the shape, as before.
 //
 // Row-major operands are handed over as their column-major transposes: D^T [N x M] = W [N x K] . X^T [K x M], with W
 // as stored ([N, K] row-major = K x N column-major) under a transpose flag.
 #include <hipblaslt/hipblaslt.h>
-
-#include <stdlib.h>
 
 #include <map>
 #include <mutex>
@@ -25,16 +21,10 @@ TIS_DEFINE_LAST_ERROR(tis_gemm_library)
 
 namespace {
 
-constexpr int kCandidates = 8;                  // algorithms the heuristic is asked for, and that are timed
-
 struct Plan {
   hipblasLtMatmulDesc_t desc;
   hipblasLtMatrixLayout_t w, x, r, c;
-  hipblasLtMatmulAlgo_t algo;                   // the one in use: the heuristic's first until the candidates are timed
-  hipblasLtMatmulAlgo_t candidates[kCandidates];
-  int n_candidates = 0;
-  int calls = 0;
-  bool timed = false;
+  hipblasLtMatmulAlgo_t algo;
 };
 
 struct DeviceState {
@@ -45,13 +35,6 @@ struct DeviceState {
 };
 
 constexpr size_t kWorkspaceBytes = 32u << 20;   // what the library may use for split reductions
-constexpr int kTimedRuns = 3;
-// A shape's candidates are timed at its first call where a call is short (few rows: decode steps, whose graphs are
-// captured at a shape's second step and keep the algorithm they were captured with), at its third call otherwise:
-// a serving run sees hundreds of row counts once or twice, and timing costs some thirty products each.
-constexpr int kTimeAtOnceRows = 256;
-constexpr int kTimeAtCall = 3;
-int g_tune = 1;                                 // 0: take the heuristic's first choice untimed
 std::mutex g_mutex;
 std::map<int, DeviceState> g_devices;
 
@@ -79,16 +62,8 @@ TIS_EXPORT int tis_gemm_library_init() {
   return device_state(&st);
 }
 
-// 0: a shape's algorithm is the library's first choice, untimed (the same from run to run)
-TIS_EXPORT int tis_gemm_library_tune(int on) {
-  std::lock_guard<std::mutex> lock(g_mutex);
-  g_tune = on ? 1 : 0;
-  return 0;
-}
-
 // R: null, or the residual added to the product (it may be C itself). A shape's first call asks the library for
-// an algorithm and must not happen under stream capture; later calls only launch (one of them, outside any capture,
-// also times the candidates: see kTimeAtCall).
+// an algorithm and must not happen under stream capture; later calls only launch.
 // out_f32: C holds 32-bit floats (the output table's logits); no residual then.
 TIS_EXPORT int tis_gemm_library(const void* X, long x_ld, const void* W, const void* R, long r_ld, void* C, long c_ld,
                                 int M, int N, int K, int out_f32, hipStream_t stream) {
@@ -117,56 +92,18 @@ TIS_EXPORT int tis_gemm_library(const void* X, long x_ld, const void* W, const v
     if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return tis_fail("gemm_library: no preference object");
     size_t ws = kWorkspaceBytes;
     hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
-    hipblasLtMatmulHeuristicResult_t found[kCandidates];
+    hipblasLtMatmulHeuristicResult_t found[1];
     int n_found = 0;
     const hipblasStatus_t hs =
-        hipblasLtMatmulAlgoGetHeuristic(st->handle, p.desc, p.w, p.x, p.r, p.c, pref, kCandidates, found, &n_found);
+        hipblasLtMatmulAlgoGetHeuristic(st->handle, p.desc, p.w, p.x, p.r, p.c, pref, 1, found, &n_found);
     hipblasLtMatmulPreferenceDestroy(pref);
     if (hs != HIPBLAS_STATUS_SUCCESS || n_found < 1)
       return tis_fail("gemm_library: the library has no algorithm for M=%d N=%d K=%d (status %d)", M, N, K, (int)hs);
-    p.n_candidates = n_found;
-    for (int i = 0; i < n_found; ++i) p.candidates[i] = found[i].algo;
     p.algo = found[0].algo;
     it = st->plans.emplace(key, p).first;
   }
-  Plan& p = it->second;
+  const Plan& p = it->second;
   const float alpha = 1.f, beta = R ? 1.f : 0.f;
-  ++p.calls;
-  if (g_tune && !p.timed && p.n_candidates > 1 && (M <= kTimeAtOnceRows || p.calls >= kTimeAtCall)) {
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    hipStreamIsCapturing(stream, &capturing);
-    void* scratch = nullptr;
-    const size_t c_bytes = (size_t)M * c_ld * (out_f32 ? 4 : 2);
-    if (capturing == hipStreamCaptureStatusNone && hipMalloc(&scratch, c_bytes) == hipSuccess) {
-      // results go to the scratch buffer, so a residual that is added in place is read but never written here
-      p.timed = true;
-      hipEvent_t t0, t1;
-      hipEventCreate(&t0);
-      hipEventCreate(&t1);
-      float best_ms = 0.f;
-      const bool log = getenv("TIS_GEMM_TUNE_LOG") != nullptr;      // the candidates' times, for a look at the choice
-      for (int i = 0; i < p.n_candidates; ++i) {
-        bool ok_run = true;
-        float t = 0.f;
-        for (int run = 0; run <= kTimedRuns && ok_run; ++run) {     // the first run is not timed
-          if (run == 1) hipEventRecord(t0, stream);
-          ok_run = hipblasLtMatmul(st->handle, p.desc, &alpha, W, p.w, X, p.x, &beta, R ? R : scratch, p.r, scratch, p.c,
-                                   &p.candidates[i], st->workspace, kWorkspaceBytes, stream) == HIPBLAS_STATUS_SUCCESS;
-        }
-        hipEventRecord(t1, stream);
-        if (hipEventSynchronize(t1) != hipSuccess || !ok_run) continue;
-        hipEventElapsedTime(&t, t0, t1);
-        if (log) fprintf(stderr, "gemm_library: M=%d N=%d K=%d candidate %d: %.1f us\n", M, N, K, i, t * 1000.f / kTimedRuns);
-        if (best_ms == 0.f || t < best_ms) {
-          best_ms = t;
-          p.algo = p.candidates[i];
-        }
-      }
-      hipEventDestroy(t0);
-      hipEventDestroy(t1);
-      hipFree(scratch);
-    }
-  }
   const hipblasStatus_t ms = hipblasLtMatmul(st->handle, p.desc, &alpha, W, p.w, X, p.x, &beta, R ? R : C, p.r, C, p.c,
                                              &p.algo, st->workspace, kWorkspaceBytes, stream);
   if (ms != HIPBLAS_STATUS_SUCCESS) return tis_fail("gemm_library: hipblasLtMatmul failed for M=%d N=%d K=%d (status %d)", M, N, K, (int)ms);

@@ -81,7 +81,6 @@ _SIGNATURES["gemm_skinny"] = ("tis_gemm_skinny", {
 })
 _SIGNATURES["gemm_library"] = ("tis_gemm_library", {
     "tis_gemm_library_init": [],
-    "tis_gemm_library_tune": [_I],
     "tis_gemm_library": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _I, _P],
 })
 _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {

@@ -487,7 +487,9 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     for (int t = 0; t < 2; ++t) {
       const int key0 = k_lo + s * 32 + t * 16;
       const int pg = __builtin_amdgcn_readfirstlane(t ? pages.y : pages.x);
-      const long page = (long)(key0 < k_hi ? pg : 0) * page_stride;
+      // (a page that a window has passed and given back reads as -1 in the table: page 0 stands in, masked like
+      // a tile past the keys)
+      const long page = (long)(key0 < k_hi && pg >= 0 ? pg : 0) * page_stride;
       const int slot0 = PS16 ? 0 : key0 % page_size;
       kbase[t] = page + (long)slot0 * HD;
       vbase[t] = page + slot0;
@@ -847,6 +849,8 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
     n_splits = 1;
   }
   if (n_tiles > 0 && group > 16 * TNB) return tis_fail("attention_mfma: a group of %d query heads does not fit a tile's wave", group);
+  if (n_tiles > 0 && 4L * n_kv_heads * page_size * HD >= (1L << 31))
+    return tis_fail("attention_mfma: a page of %d key/value heads x %d slots is too large for the tile kernel's 32-bit offsets", n_kv_heads, page_size);
   if (n_tiles == 0) tile_splits = 1;
   if (page_size < 16 || page_size % 16) return tis_fail("attention_mfma: page size %d is no multiple of 16", page_size);
   if (n_splits < 1 || n_splits > 65535 || tile_splits < 1 || tile_splits > 65535 || n_kv_heads > 65535)

@@ -67,3 +67,36 @@ def test_graph_survives_changing_batches(max_graphs):
     assert min(3, max_graphs) <= len(eng._graphs) <= max_graphs and eng.graph_replays >= 30
     H.compare_with_plain(folder, reqs, main, {}, 2e-2 * max(1.0, max(
         H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values())), 0)
+
+
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_repeated_prompt_steps_are_replayed(name):
+    """A step of the same shape (two prompts of fixed lengths in one batch, the same places wanted) comes again and
+    again with other tokens, in other slots and pages, with eager steps of other shapes in between: from its third
+    occurrence it is replayed from a graph, and every occurrence must match the plain implementation."""
+    folder = H.model_folder(name, "bfloat16")
+    vocab = H.TINY[name]["cfg"].vocab_size
+    eng = Engine(folder, dtype="bfloat16", page_size=H.TINY[name]["page_size"], max_tokens=512, max_requests=8)
+    lengths = (41, 30)
+    worst_scale = 1.0
+    for rep in range(7):
+        reqs = {f"p{rep}_{i}": H.random_ids(vocab, n, 300 + 10 * rep + i) for i, n in enumerate(lengths)}
+        if rep % 2:
+            # something else lives in the cache meanwhile, so slots and pages differ from the captured step's
+            eng.step([("other", H.random_ids(vocab, 13 + rep, 77), [0])])
+        out = eng.step([(rid, ids, [0, len(ids) // 2, len(ids) - 1]) for rid, ids in reqs.items()])
+        lg = out.logits.float().cpu().clone()
+        torch.cuda.synchronize()
+        main = {}
+        for k, (rid, ids) in enumerate(reqs.items()):
+            for j, p in enumerate((0, len(ids) // 2, len(ids) - 1)):
+                main[(rid, p)] = lg[3 * k + j]
+        scale = max(1.0, max(H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values()))
+        H.compare_with_plain(folder, reqs, main, {}, 2e-2 * scale, 0)
+        for rid in reqs:
+            eng.close(rid)
+        if rep % 2:
+            eng.close("other")
+    assert eng.graph_replays >= 4
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()

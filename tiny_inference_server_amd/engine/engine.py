@@ -168,14 +168,18 @@ class Engine:
             slot, fed = self.requests[rid]
             self.cache.grow(slot, fed + len(toks))
             batch_entries.append(Entry(slot, fed, arrays[rid], list(want)))
-        logits = None
-        if (self.use_graphs and not heads and
-                all(len(e.tokens) == 1 and e.start >= self.model.max_lag and list(e.want) == [0]
-                    for e in batch_entries)):
-            logits = self._decode_step(batch_entries)
+        logits = plan = None
+        if self.use_graphs and not heads:
+            if all(len(e.tokens) == 1 and e.start >= self.model.max_lag and list(e.want) == [0] for e in batch_entries):
+                logits = self._decode_step(batch_entries)
+            else:
+                logits, plan = self._repeated_step(batch_entries)
         if logits is None:
-            step = build_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
-                                    self.device, self.spec.max_context, getattr(self.ops, "plan_rows", None))
+            if plan is not None:
+                step = materialize(plan, self.device)
+            else:
+                step = build_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
+                                        self.device, self.spec.max_context, getattr(self.ops, "plan_rows", None))
             outs = self.model.forward(step, self.cache)
         n = sum(len(e.want) for e in batch_entries)
         vocab = self.spec.vocab_size
@@ -204,6 +208,35 @@ class Engine:
             self.cache.release_behind(slot, fed + len(toks), self.model.max_lag)
         return StepOutput(logits, head_logits, head_valid)
 
+    def _repeated_step(self, batch_entries):
+        """Any other step whose shape has come before: the same requests' row counts, the same places wanted, the
+        same work for the attention kernels (a batch of equal prompts, a benchmark's prefill). Returns (logits or
+        None, the step's plan); from its third occurrence on a shape is replayed from a captured graph."""
+        from .graph import DecodeGraph
+        pages = max((max(len(g.tables[e.slot]) for e in batch_entries) for g in self.cache.groups.values()), default=1)
+        width = -(-pages // self.graph_table_pages) * self.graph_table_pages
+        plan = plan_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
+                               self.spec.max_context, getattr(self.ops, "plan_rows", None), table_width=width)
+        # what the host decides from, beyond the arrays' shapes
+        key = ("step", width, plan.layout(),
+               tuple((pl["max_rows"], pl["keep_count"], pl["previous_rows"], tuple(pl["valid"])) for pl in plan.plans))
+        graph = self._graphs.get(key)
+        if graph is None:
+            if len(self._graph_seen) > 4096:          # shapes that never came back
+                self._graph_seen.clear()
+            seen = self._graph_seen.get(key, 0)
+            self._graph_seen[key] = seen + 1
+            if seen < 2:
+                return None, plan
+            if len(self._graphs) >= self.max_graphs:
+                torch.cuda.synchronize(self.device)
+                self._graphs.popitem(last=False)
+            graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size)
+        else:
+            self._graphs.move_to_end(key)
+        self.graph_replays += 1
+        return graph.run(plan), plan
+
     def _decode_step(self, batch_entries):
         """A step of single tokens through a captured graph: logits [requests, vocab], valid until the next step."""
         from .graph import DecodeGraph
@@ -225,8 +258,8 @@ class Engine:
             seen = self._graph_seen.get(key, 0)
             self._graph_seen[key] = seen + 1
             if seen == 0:
-                # the first step of a shape runs as it is: it warms the library's choices for these shapes and
-                # sizes the kernels' workspace, so the capture that follows records kernel launches only
+                # the first step of a shape runs as it is: it warms the library's choices for these shapes, so the
+                # capture that follows records kernel launches only
                 step = materialize(plan, self.device)
                 for st in step.stages:
                     st.max_kv_len = width * self.page_size

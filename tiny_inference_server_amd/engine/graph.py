@@ -1,13 +1,14 @@
-"""Captured decode steps.
+"""Captured steps.
 
 A step in which every request brings exactly one token, far enough into its sequence that every stage has
 one row per request, always launches the same kernels on arrays of the same shapes. Such a step is
 captured once per (number of requests, block-table width) as a HIP graph over a fixed device buffer that
 holds the step's integer arrays; later steps of the same shape copy their arrays into that buffer and
-replay the graph, which removes the launch cost of several hundred small kernels.
+replay the graph, which removes the launch cost of several hundred small kernels. Any other step is captured
+the same way once its exact shape (row counts, wanted places, attention work) has come three times.
 
-Nothing is cleared inside the graph with a memset, and the first step of a shape runs without a graph (it
-also sizes the kernels' workspace), so a capture records kernel launches only.
+Nothing is cleared inside the graph with a memset, and the first steps of a shape run without a graph (the
+library chooses its algorithms for the shape then), so a capture records kernel launches only.
 """
 from __future__ import annotations
 
@@ -25,14 +26,17 @@ class DecodeGraph:
         self.dev = torch.zeros(max(plan.packer.total, 4), dtype=torch.int32, device=dev)
         self.copied = torch.cuda.Event()
         self.step = materialize(plan, dev, self.host, self.dev)
-        for st in self.step.stages:
+        for st in self.step.stages:          # later steps of the shape may see more keys than this one
             st.max_kv_len = kv_capacity
         n = self.step.n_wanted
         self.graph = torch.cuda.CUDAGraph()
         torch.cuda.synchronize(dev)
         with torch.cuda.graph(self.graph):
             outs = engine.model.forward(self.step, engine.cache)
-            self.logits = engine.model.logits(outs[0].hidden, self.step.stages[0].want_index, n)
+            if n:
+                self.logits = engine.model.logits(outs[0].hidden, self.step.stages[0].want_index, n)
+            else:
+                self.logits = torch.empty(0, engine.spec.vocab_size, dtype=torch.float32, device=dev)
         self.copied.record()
         # what the quick update needs: which requests, in which order, the buffer holds, and where their arrays lie
         self.slots = tuple(e.slot for e in plan.entries)

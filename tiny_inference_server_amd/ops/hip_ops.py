@@ -215,7 +215,9 @@ class HipOps:
                 self.gemm_library.tis_gemm_library_init()
         self._attn_groups = set()          # group sizes of the attention mixers built on these ops
         self._attn_mfma = {}               # head size -> library
-        self._workspace = None
+        # partial results of split key ranges: one buffer of fixed size that never moves (captured graphs hold its address)
+        self._workspace = torch.empty(_ATTN_WORKSPACE_FLOATS, dtype=torch.float32, device=self.device) \
+            if dtype == torch.bfloat16 else None
 
     # ---- planning on the host --------------------------------------------------------------------------
     def register_attention(self, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
@@ -586,17 +588,13 @@ class HipOps:
                 share = tile_steps * n_kv_heads / _ATTN_TILE_GROUPS
                 tile_min_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
                 tile_splits = max(1, -(-batch.max_kv_len // 32) // tile_min_steps)
-            # partial results of split key ranges live in one workspace of fixed size, allocated once and never
-            # moved (captured graphs hold its address); fewer splits where it would not suffice
+            # partial results of split key ranges live in one workspace of fixed size; fewer splits where it
+            # would not suffice
             most = max(1, (_ATTN_WORKSPACE_FLOATS - n) // (n * n_heads * (head_dim + 2)))
             n_splits, tile_splits = min(n_splits, most), min(tile_splits, most)
             stride = max(n_splits, tile_splits)
             part_o = part_ml = row_splits = None
             if stride > 1:
-                if self._workspace is None:
-                    if torch.cuda.is_current_stream_capturing():
-                        raise KernelError("the attention workspace must exist before a graph is captured")
-                    self._workspace = torch.empty(_ATTN_WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
                 part_o = self._workspace
                 part_ml = self._workspace[n * n_heads * stride * head_dim:]
                 if not single:

@@ -373,6 +373,40 @@ def test_rope_and_cache_write(ops_for, dtype, n_heads, n_kv, hd, page_size, inte
     assert torch.equal(before, pa)
 
 
+@pytest.mark.parametrize("n", [23, 64, 203])
+@pytest.mark.parametrize("n_heads,n_kv,hd,page_size", [(12, 3, 128, 16), (3, 1, 64, 32), (5, 5, 48, 16), (2, 1, 256, 16)])
+def test_rope_and_cache_write_of_pair_ordered_rows(ops_for, n_heads, n_kv, hd, page_size, n):
+    """Rows as the fused q/k/v projection leaves them (the members of every rotary pair side by side): few rows, and
+    enough for the kernel that takes sixteen rows a workgroup and turns the values through LDS. Slots are runs of
+    consecutive positions that start mid-page, with one row out of line, as the rows of prompt portions are."""
+    ops, ref = ops_for(torch.bfloat16), TorchOps(dtype=torch.bfloat16)
+    dtype = torch.bfloat16
+    n_pages, max_ctx = 40, 700
+    j = torch.arange(hd // 2)
+    theta = 1.0 / torch.pow(torch.tensor(10000.0), (2 * j.float()) / hd)
+    ang = torch.outer(torch.arange(max_ctx).float(), theta)
+    table = torch.stack((torch.cos(ang), torch.sin(ang)), -1).contiguous()
+    qkv = rnd((n, (n_heads + 2 * n_kv) * hd), dtype, 54)
+    first = 5
+    positions = torch.arange(first, first + n, dtype=torch.int32)
+    pages = random.Random(55).sample(range(n_pages), -(-(first + n) // page_size) + 1)
+    slots = torch.tensor([pages[p // page_size] * page_size + p % page_size for p in positions.tolist()], dtype=torch.int32)
+    slots[n // 2], positions[n // 2] = pages[-1] * page_size + 3, 650          # a row of another request in between
+    plane0 = rnd((n_pages, 2, n_kv, page_size, hd), dtype, 56)
+    for write_cache in (True, False):
+        pa, pb = plane0.clone().cuda(), plane0.clone()
+        qa = torch.zeros(n, n_heads * hd, dtype=dtype).cuda()
+        qb = torch.zeros(n, n_heads * hd, dtype=dtype)
+        ops.rope_write_kv(qkv.clone().cuda(), positions.cuda(), slots.cuda(), table.cuda(), pa, n_heads, n_kv, hd,
+                          page_size, False, write_cache=write_cache, paired=True, q_out=qa)
+        ref.rope_write_kv(qkv.clone(), positions, slots, table, pb, n_heads, n_kv, hd, page_size, False,
+                          write_cache=write_cache, paired=True, q_out=qb)
+        torch.testing.assert_close(qa.cpu().float(), qb.float(), **tol(dtype))
+        torch.testing.assert_close(pa.cpu().float(), pb.float(), **tol(dtype))
+        if not write_cache:
+            assert torch.equal(pa.cpu(), plane0)
+
+
 @pytest.mark.parametrize("V", [6, 100, 1000, 48000])
 def test_sampling(ops_for, V):
     ops, ref = ops_for(torch.float32), TorchOps()

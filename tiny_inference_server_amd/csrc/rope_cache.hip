@@ -80,6 +80,75 @@ __global__ __launch_bounds__(RC_THREADS) void rope_write_kv_kernel(T* __restrict
   }
 }
 
+// The same for many rows of a pair-ordered bfloat16 projection (a prompt portion), sixteen rows a workgroup.
+// Queries and keys: a lane takes four pairs (16 bytes in, two 8-byte runs out), so a wave does four (row, head)
+// items an instruction instead of one. Values: the sixteen rows of a head pass through LDS and leave transposed,
+// lanes side by side along the rows: rows of a portion have consecutive slots, so a wave's 2-byte stores fall
+// into runs of up to 32 bytes ([head_dim][slot] keeps a page's slots of one element together) instead of
+// sixty-four separate places.
+static constexpr int RB = 16;            // rows of a workgroup
+typedef __attribute__((ext_vector_type(8))) __bf16 rc_bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 rc_bf16x4;
+
+__global__ __launch_bounds__(RC_THREADS) void rope_write_kv_rows_kernel(
+    const bf16* __restrict__ qkv, long ld, const int* __restrict__ positions, const int* __restrict__ write_slots,
+    const float2* __restrict__ table, bf16* __restrict__ plane, int rows, int n_heads, int n_kv_heads, int head_dim,
+    int page_size, int write_cache, bf16* __restrict__ q_out, long q_out_ld) {
+  __shared__ bf16 tile[RB][256 + 8];      // one head of sixteen rows; head sizes up to 256
+  const long r0 = (long)blockIdx.x * RB;
+  const int n_rows = (int)min((long)RB, rows - r0);
+  const int half = head_dim / 2, pieces = head_dim / 8;     // a piece: four pairs, 16 bytes
+  const int rotated = n_heads + (write_cache ? n_kv_heads : 0);
+  // queries and keys of this workgroup's share of the heads: piece after piece over (head, row, piece)
+  for (int hh = blockIdx.y; hh < rotated; hh += gridDim.y) {
+    for (int i = threadIdx.x; i < n_rows * pieces; i += RC_THREADS) {
+      const int row = i / pieces, piece = i % pieces;
+      const long r = r0 + row;
+      const rc_bf16x8 x = *reinterpret_cast<const rc_bf16x8*>(qkv + r * ld + (long)hh * head_dim + piece * 8);
+      const float4* cs = reinterpret_cast<const float4*>(table + (long)positions[r] * half + piece * 4);
+      const float4 cs01 = cs[0], cs23 = cs[1];
+      const float c[4] = {cs01.x, cs01.z, cs23.x, cs23.z}, sn[4] = {cs01.y, cs01.w, cs23.y, cs23.w};
+      rc_bf16x4 y1, y2;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float x1 = static_cast<float>(x[2 * e]), x2 = static_cast<float>(x[2 * e + 1]);
+        y1[e] = static_cast<__bf16>(x1 * c[e] - x2 * sn[e]);
+        y2[e] = static_cast<__bf16>(x2 * c[e] + x1 * sn[e]);
+      }
+      bf16* dst;
+      if (hh < n_heads) {
+        dst = q_out + r * q_out_ld + (long)hh * head_dim;
+      } else {
+        const int slot = write_slots[r];
+        dst = plane + (((long)(slot / page_size) * 2) * n_kv_heads + (hh - n_heads)) * page_size * head_dim +
+              (long)(slot % page_size) * head_dim;
+      }
+      *reinterpret_cast<rc_bf16x4*>(dst + piece * 4) = y1;
+      *reinterpret_cast<rc_bf16x4*>(dst + half + piece * 4) = y2;
+    }
+  }
+  if (!write_cache) return;
+  // values
+  const int row_t = threadIdx.x % RB, d_t = threadIdx.x / RB;          // on the way out: rows side by side
+  long v_dst = 0;
+  if (row_t < n_rows) {
+    const int slot = write_slots[r0 + row_t];
+    v_dst = ((long)(slot / page_size) * 2 + 1) * n_kv_heads * page_size * head_dim + slot % page_size;
+  }
+  for (int kvh = blockIdx.y; kvh < n_kv_heads; kvh += gridDim.y) {
+    __syncthreads();                                                     // the tile's last readers are done
+    for (int i = threadIdx.x; i < n_rows * pieces; i += RC_THREADS) {
+      const int row = i / pieces, piece = i % pieces;
+      *reinterpret_cast<rc_bf16x8*>(&tile[row][piece * 8]) = *reinterpret_cast<const rc_bf16x8*>(
+          qkv + (r0 + row) * ld + (long)(n_heads + n_kv_heads + kvh) * head_dim + piece * 8);
+    }
+    __syncthreads();
+    if (row_t < n_rows)
+      for (int d = d_t; d < head_dim; d += RC_THREADS / RB)
+        plane[v_dst + ((long)kvh * head_dim + d) * page_size] = tile[row_t][d];
+  }
+}
+
 TIS_EXPORT int tis_rope_write_kv(int dtype, void* qkv, long ld, const int* positions, const int* write_slots,
                                  const float* table, void* plane, int rows, int n_heads, int n_kv_heads, int head_dim,
                                  int page_size, int interleaved, int write_cache, int paired, void* q_out,
@@ -90,6 +159,16 @@ TIS_EXPORT int tis_rope_write_kv(int dtype, void* qkv, long ld, const int* posit
                     n_kv_heads, head_dim, page_size);
   if (paired && !q_out) return tis_fail("rope_write_kv: paired input needs a separate output for the queries");
   const int total_heads = n_heads + 2 * n_kv_heads;
+  if (dtype == TIS_BF16 && paired && !interleaved && table && rows >= 4 * RB && head_dim % 8 == 0 && head_dim <= 256 &&
+      ld % 8 == 0 && q_out_ld % 4 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)q_out % 8) == 0 &&
+      (!write_cache || (uintptr_t)plane % 8 == 0)) {
+    dim3 grid((rows + RB - 1) / RB, std::min(total_heads, 4));
+    rope_write_kv_rows_kernel<<<grid, RC_THREADS, 0, stream>>>((const bf16*)qkv, ld, positions, write_slots,
+                                                              (const float2*)table, (bf16*)plane, rows, n_heads,
+                                                              n_kv_heads, head_dim, page_size, write_cache,
+                                                              (bf16*)q_out, q_out_ld);
+    return tis_launch_status("rope_write_kv_rows");
+  }
   // measured on MI355X with 18 heads of 128: few rows like their heads spread wide (64 rows: 3.5 us over five
   // workgroups a row against 4.5 over one), thousands of rows like two workgroups a row (10.3 against 11.1 us)
   const int wide = (total_heads + RC_THREADS / 64 - 1) / (RC_THREADS / 64);

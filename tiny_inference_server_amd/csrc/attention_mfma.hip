@@ -1,7 +1,9 @@
 // Attention over paged keys and values on the matrix cores (bfloat16, gfx950), for decode rows and for
 // portions of prompts alike. Compiled for one head size: -DTIS_HD=<multiple of 16, at most 256>.
+// Two kernels and a merge: the wave kernel described next, and further down the tile kernel that takes long
+// portions (a workgroup of four waves sharing keys and values through LDS).
 //
-// One wavefront owns an *item*: up to 16*NB query columns that share a request and a key/value head, a
+// Wave kernel. One wavefront owns an *item*: up to 16*NB query columns that share a request and a key/value head, a
 // column being (row, query head): n_rows consecutive positions of the request times the group's query heads.
 // A decode row is an item of one row; all query heads of its group share one pass over the keys, so keys
 // and values are read once per group, not once per query head. A long key range is cut into splits that
@@ -17,7 +19,7 @@
 //                                              bfloat16 (as the reference does before P.V:
 //                                              paged_attention_kernels.py:108), exactly as S^T left it in registers
 // Both products put the column on the lane, so the softmax statistics never cross lanes except for the
-// reduction over the four key groups, and no LDS is used. Masked keys are read (their page is mapped), but their
+// reduction over the four key groups, and this kernel uses no LDS. Masked keys are read (their page is mapped), but their
 // scores are replaced by -inf and their values by zero before either is used in arithmetic, so what an earlier
 // owner left in a page never reaches a result.
 #include <type_traits>

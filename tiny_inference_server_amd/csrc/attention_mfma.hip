@@ -381,7 +381,7 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     const bf16* __restrict__ q, long q_ld, const bf16* __restrict__ plane, const int* __restrict__ block_tables,
     int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ tiles,
     bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
-    int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits, int min_steps,
+    int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits, int max_steps,
     int split_stride, int* __restrict__ row_splits) {
   constexpr int NB = TNB;
   __shared__ __attribute__((aligned(16))) bf16 k_lds[TBUF][TCH * 8];
@@ -430,8 +430,8 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   const int k_lo = t_lo & ~31;
   const int k_hi = tp_last + 1;
   const int n_steps = (k_hi - k_lo + 31) / 32;
-  int item_splits = n_splits;
-  if (min_steps > 0) item_splits = max(1, min(n_splits, n_steps / min_steps));
+  // as many splits as keep each no longer than max_steps (the host's bound on the chain of steps one workgroup walks)
+  const int item_splits = max(1, min(n_splits, (n_steps + max_steps - 1) / max_steps));
   if (split >= item_splits) return;                   // the whole workgroup, before any barrier
   if (row_splits && kvh == 0 && split == 0 && tid < t_rows) row_splits[t_row0 + tid] = item_splits;
   const int per_split = (n_steps + item_splits - 1) / item_splits;
@@ -829,15 +829,15 @@ TIS_EXPORT int tis_attention_mfma_tile_columns() { return 16 * TNB; }
 // rows * group_size <= 16 * nb. Null: n_items single rows, item i being row i. tiles: (first row, rows) pairs for the
 // workgroup kernel, rows <= 4 * (tis_attention_mfma_tile_columns() / group_size); items and tiles together hold every row once.
 // n_splits / tile_splits: what the grid offers an item / a tile. part_o / part_ml: workspace where either exceeds
-// one, [rows][heads][S][HD] floats and [rows][heads][S] float pairs, S the larger of the two. min_steps > 0 (tiles:
-// tile_min_steps): an item uses min(n_splits, its steps of 32 keys / min_steps) splits, and row_splits [rows]
-// receives each row's count.
+// one, [rows][heads][S][HD] floats and [rows][heads][S] float pairs, S the larger of the two. min_steps > 0: an item
+// uses min(n_splits, its steps of 32 keys / min_steps) splits; a tile uses as many as keep each at most
+// tile_max_steps long; row_splits [rows] receives each row's count.
 TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
                                   const int* row_seq, const int* positions, const int* items, int n_items, int nb,
                                   const int* tiles, int n_tiles, void* out, long out_ld, float* part_o,
                                   float* part_ml, int rows, int n_heads, int n_kv_heads, int head_dim, int page_size,
                                   int window, float scale, int n_splits, int min_steps, int tile_splits,
-                                  int tile_min_steps, int* row_splits, hipStream_t stream) {
+                                  int tile_max_steps, int* row_splits, hipStream_t stream) {
   if ((n_items == 0 && n_tiles == 0) || rows == 0) return 0;
   if (n_items < 0 || n_tiles < 0 || (n_tiles > 0 && !tiles)) return tis_fail("attention_mfma: bad item counts %d, %d", n_items, n_tiles);
   if (head_dim != HD) return tis_fail("attention_mfma: built for head size %d, called with %d", HD, head_dim);
@@ -861,7 +861,8 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
   if (stride > 1 && (!part_o || !part_ml)) return tis_fail("attention_mfma: %d splits need a workspace", stride);
   if (min_steps < 0 || (min_steps > 0 && n_splits > 1 && !row_splits))
     return tis_fail("attention_mfma: splits chosen item by item (min_steps=%d) need the per-row count array", min_steps);
-  if (n_tiles > 0 && stride > 1 && (tile_min_steps < 1 || !row_splits || (n_items > 0 && min_steps < 1)))
+  if (n_tiles > 0 && tile_max_steps < 1) return tis_fail("attention_mfma: a tile's splits need a longest chain of at least one step");
+  if (n_tiles > 0 && stride > 1 && (!row_splits || (n_items > 0 && min_steps < 1)))
     return tis_fail("attention_mfma: tiles beside split key ranges need the per-row count array and a minimum of steps");
   if (stride == 1 || (n_tiles == 0 && min_steps == 0)) row_splits = nullptr;
   if ((q_ld % 8) || (out_ld % 4) || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)plane % 16))
@@ -894,7 +895,7 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
   attention_tile_kernel<PSV><<<grid, TW * 64, 0, stream>>>(                                                      \
       (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)tiles,     \
       (bf16*)out, out_ld, part_o, (float2*)part_ml, group, n_kv_heads, n_heads, page_size, window, scale_log2,   \
-      tile_splits, tile_min_steps, stride, row_splits)
+      tile_splits, tile_max_steps, stride, row_splits)
     if (page_size == 16) LAUNCH(true);
     else LAUNCH(false);
 #undef LAUNCH

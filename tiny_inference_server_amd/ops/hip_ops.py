@@ -111,8 +111,11 @@ _ATTN_MIN_SPLIT_KEYS = 128      # a split shorter than this costs more in mergin
 _ATTN_TILE_WAVES = 4            # waves of the workgroup that takes a tile of a long portion
 _ATTN_TILE_GROUPS = 512         # workgroups of the tile kernel that the chip runs side by side
 _ATTN_TILE_MIN_STEPS = 8        # steps of 32 keys below which a tile's split is not worth its merge
-_ATTN_TILE_SPLIT_SLACK = 1.5    # a split may be this much longer than an even share of all steps
-_ATTN_TILE_MIN_WORK = 4000      # tile steps times key/value heads below which the one-wave kernel is the faster
+_ATTN_TILE_SPLIT_SLACK = 1.4    # a split may be this much longer than an even share of all steps
+_ATTN_TILE_PARTIAL_BYTES = 40 << 20   # partial results (32-bit, per split) beyond which the merge costs more than
+                                      # shorter chains save; at least two splits are always allowed
+_ATTN_TILE_MIN_WORK = 3000      # tile steps times key/value heads below which the one-wave kernel is the faster ...
+_ATTN_TILE_MIN_WORK_MIXED = 1500   # ... and beside decoded tokens deep in their requests (their splits are merged anyway)
 _ATTN_WORKSPACE_FLOATS = 16 << 20
 
 
@@ -125,14 +128,17 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
     """Work items of the matrix-core attention kernels for the rows of one stage.
 
     seq_rows: (first row, first position, rows) per request. Returns (column blocks per item, items, tiles, steps):
-    items and tiles are int32 arrays of (first row, rows) lines that together hold every row once, steps is the
-    number of 32-key steps that all tiles walk together (the kernel's work, by which its key splits are sized).
+    items and tiles are int32 arrays of (first row, rows) lines that together hold every row once, steps is
+    (the number of 32-key steps that all tiles walk together, the most that one tile walks): the kernel's work, by
+    which its key splits are sized.
     An item (one wave) holds consecutive rows of one request, rows * group_size <= 16 * blocks. When no request has
     more than one row the list is simply every row in order, which the kernel knows without being given a list.
     A tile (a workgroup of four waves, `tile_cols` columns each; 0: no tiles) takes up to 4 * (tile_cols // group_size)
     consecutive rows of a portion that fills at least half of one. Tiles are made only where their steps times
     `n_kv_heads` (the workgroups' work) reach _ATTN_TILE_MIN_WORK (0: always): a tile's waves walk its keys in
-    lockstep, which pays when there is work for every compute unit and costs on a short prompt.
+    lockstep, which pays when there is work for every compute unit and costs on a short prompt. Measured at 12 heads
+    of 128 over 3 (tiles / one-wave kernel, us): 1,536 rows 40 / 48, 1,024 rows 32 / 29, three portions of 700 rows
+    39 / 34; a portion of 512 rows at 1,000 beside 8 decoded tokens 53 / 65, one of 256 rows 41 / 29.
     """
     none = np.zeros((0, 2), dtype=np.int32)
     single = all(n <= 1 for _, _, n in seq_rows)
@@ -140,20 +146,21 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
         nb = 1
         while group_size > 16 * nb:
             nb *= 2
-        return nb, np.asarray([(first, 1) for first, _, n in seq_rows if n], dtype=np.int32).reshape(-1, 2), none, 0
+        return nb, np.asarray([(first, 1) for first, _, n in seq_rows if n], dtype=np.int32).reshape(-1, 2), none, (0, 0)
     tile_rows = _ATTN_TILE_WAVES * (tile_cols // group_size)
     tiled = [(f, p0, n) for f, p0, n in seq_rows if tile_rows and n >= max(2, tile_rows // 2)]
     if tiled and n_kv_heads:
         work = sum(int(((p0 + np.minimum(np.arange(0, n, tile_rows) + tile_rows, n) + 31) // 32).sum())
                    for _, p0, n in tiled) * n_kv_heads
-        if work < _ATTN_TILE_MIN_WORK:
+        deep = any(n == 1 and p0 >= 512 for _, p0, n in seq_rows)
+        if work < (_ATTN_TILE_MIN_WORK_MIXED if deep else _ATTN_TILE_MIN_WORK):
             tiled = []
     taken = {f for f, _, _ in tiled}
     rest = [(f, p0, n) for f, p0, n in seq_rows if n > 0 and f not in taken]
 
     def cut(segments, per_item):
         if not segments:
-            return none, 0
+            return none, (0, 0)
         firsts, counts, keys = [], [], []
         for first, p0, n in segments:
             r = np.arange(0, n, per_item, dtype=np.int64)
@@ -165,7 +172,8 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
         # those with the most keys first: under a causal mask the last rows of a prompt are the longest, and
         # started last they would run on alone while the rest of the chip idles
         order = np.argsort(-keys, kind="stable")
-        return np.stack((firsts[order], counts[order]), axis=1).astype(np.int32), int(((keys + 31) // 32).sum())
+        steps = (keys + 31) // 32
+        return np.stack((firsts[order], counts[order]), axis=1).astype(np.int32), (int(steps.sum()), int(steps.max()))
 
     nb = 2
     # 64-column items halve what a portion reads of its keys and values; they pay once there are enough of them
@@ -571,7 +579,7 @@ class HipOps:
                     raise KernelError(f"attention: the kernel's tiles hold {built} columns a wave, the planner "
                                       f"assumes {cols}")
             single = items is None and n_tiles == 0
-            n_splits, min_steps, tile_splits, tile_min_steps = 1, 0, 1, _ATTN_TILE_MIN_STEPS
+            n_splits, min_steps, tile_splits, tile_max_steps = 1, 0, 1, 1 << 20
             if n_items:
                 # decoded tokens: every request's keys are cut into the same number of splits, enough to spread a
                 # short batch over the chip. Prompt rows: the grid offers more splits than the chip needs and every
@@ -583,11 +591,16 @@ class HipOps:
                 n_splits = max(1, min(-(-target // (n_items * n_kv_heads)), batch.max_kv_len // min_keys))
                 min_steps = 0 if single else _ATTN_PROMPT_MIN_STEPS
             if n_tiles:
-                # a tile's keys are cut where it alone would run longer than an even share of all tiles' steps
-                # (the last rows of a long prompt); a split is never shorter than _ATTN_TILE_MIN_STEPS
-                share = tile_steps * n_kv_heads / _ATTN_TILE_GROUPS
-                tile_min_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
-                tile_splits = max(1, -(-batch.max_kv_len // 32) // tile_min_steps)
+                # a tile's keys are cut so that no workgroup walks a chain of steps much longer than an even share of
+                # all tiles' steps: the last rows of a long prompt would otherwise run on alone. Measured at 12 heads
+                # of 128 (tiles / one-wave kernel, us): 2,048 rows from 0: 54 / 69; from 2,048: 99 / 134; from 6,144:
+                # 196 / 260; 4,096 rows: 146 / 202.
+                all_steps, longest = tile_steps
+                share = all_steps * n_kv_heads / _ATTN_TILE_GROUPS
+                tile_max_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
+                most_splits = max(2, _ATTN_TILE_PARTIAL_BYTES // (n * n_heads * head_dim * 4))
+                tile_splits = max(1, min(most_splits, -(-longest // tile_max_steps)))
+                tile_max_steps = max(tile_max_steps, -(-longest // tile_splits))
             # partial results of split key ranges live in one workspace of fixed size; fewer splits where it
             # would not suffice
             most = max(1, (_ATTN_WORKSPACE_FLOATS - n) // (n * n_heads * (head_dim + 2)))
@@ -603,7 +616,7 @@ class HipOps:
                                    _ptr(batch.row_seq), _ptr(batch.positions), _ptr(items), n_items, nb, _ptr(tiles),
                                    n_tiles, _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), n, n_heads,
                                    n_kv_heads, head_dim, page_size, int(window), float(scale), n_splits, min_steps,
-                                   tile_splits, tile_min_steps, _ptr(row_splits), self._stream())
+                                   tile_splits, tile_max_steps, _ptr(row_splits), self._stream())
             return out
         self.attn_generic.tis_attention_generic(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),

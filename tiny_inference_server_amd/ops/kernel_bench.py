@@ -2,10 +2,13 @@
 
     python -m tiny_inference_server_amd.ops.kernel_bench attention --segments 0:2048
     python -m tiny_inference_server_amd.ops.kernel_bench attention --segments 4095:1x8
+    python -m tiny_inference_server_amd.ops.kernel_bench attention --segments 0:2048 --no-tiles
     python -m tiny_inference_server_amd.ops.kernel_bench product --rows 8 --out 8192 --in 1536 --kind norm+gate
 
 A segment is `first position:rows`, `xN` repeats it for N requests; `4095:1x8` is a decode step of 8 requests at
-context 4096, `0:2048` a prompt of 2,048 tokens, `4095:1x8,1000:256` a mixed step. The kernel is captured into a
+context 4096, `0:2048` a prompt of 2,048 tokens, `4095:1x8,1000:256` a mixed step. Long portions go to the
+workgroup (tile) kernel where the engine would send them; `--tiles` sends them there however little work they are,
+`--no-tiles` keeps every row with the one-wave kernel. The kernel is captured into a
 graph of `--reps` launches and the graph is timed, so host launch cost stays out. A kernel alone runs on warm caches:
 decisions about decode kernels are taken on whole decode steps (bench.py), this is for counters and first looks.
 """

@@ -1,0 +1,104 @@
+"""Steps kept in fixed buffers (the host side of captured graphs), run on the CPU stand-in for the kernels.
+
+A captured decode step keeps its integer arrays in one buffer; while the same requests come again in the same order
+only tokens, positions, write slots and newly taken pages are rewritten. "The same requests" must mean the requests
+themselves: a cache slot is handed to request after request, and a successor that holds no more pages than its
+predecessor did would otherwise run on the predecessor's block table (the policy being followed: finished requests
+leave, queued ones take their places, reference server.py:286-292).
+"""
+import pytest
+import torch
+
+import helpers as H
+from tiny_inference_server_amd.engine import Engine
+from torch_ops import TorchOps
+
+TOL = {"float32": 2e-5, "bfloat16": 2e-2}
+
+
+def engine_for(name, dtype, max_tokens, max_requests, graphs=True):
+    folder = H.model_folder(name, "float32" if dtype == "float32" else "bfloat16")
+    ops = TorchOps(dtype=torch.float32 if dtype == "float32" else torch.bfloat16, graphs=graphs)
+    return folder, Engine(folder, dtype=dtype, page_size=H.TINY[name]["page_size"], max_tokens=max_tokens,
+                          max_requests=max_requests, ops=ops)
+
+
+def scale_of(folder, reqs):
+    return max(1.0, max(H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values()))
+
+
+def one_after_the_other(reqs, prompt):
+    """Every request alone: `prompt` tokens in one step, the rest one by one; the next request starts when it ends."""
+    steps = []
+    for rid, ids in reqs.items():
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": ids[:prompt], "want": [prompt - 1]}], "end": []})
+        for p in range(prompt, len(ids)):
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": [ids[p]], "want": [0]}],
+                          "end": [rid] if p == len(ids) - 1 else []})
+    return steps
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("D", "bfloat16")])
+def test_a_slot_that_changes_hands_gets_its_new_owners_pages(name, dtype):
+    """One slot only, so every request follows its predecessor into it; the second is shorter than the first and the
+    third longer, and all decode through the same captured shape."""
+    vocab = H.TINY[name]["cfg"].vocab_size
+    reqs = {f"s{i}": H.random_ids(vocab, n, 90 + i) for i, n in enumerate([70, 40, 75, 41])}
+    folder, eng = engine_for(name, dtype, max_tokens=256, max_requests=1)
+    assert eng.use_graphs
+    main, _ = H.run_trace(eng, one_after_the_other(reqs, 9), heads=False)
+    assert eng.graph_replays > 100
+    wanted = {(rid, p) for rid, ids in reqs.items() for p in range(8, len(ids))}
+    assert set(main) == wanted
+    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()
+
+
+def test_quick_update_is_refused_after_a_slot_changed_hands():
+    """The buffer of a captured step answers for the requests it was filled with, not for their slots."""
+    name = "A"
+    vocab = H.TINY[name]["cfg"].vocab_size
+    folder, eng = engine_for(name, "float32", max_tokens=256, max_requests=1)
+    a, b = H.random_ids(vocab, 70, 1), H.random_ids(vocab, 30, 2)
+    eng.step([("a", a[:60], [])])
+    for p in range(60, 64):
+        eng.step([("a", [a[p]], [0])])
+    graph = next(iter(eng._graphs.values()))
+    slot_a = eng.requests["a"][0]
+    held = graph.occupants
+    assert graph.holds(held)
+    eng.close("a")
+    eng.step([("b", b[:20], [])])
+    assert eng.requests["b"][0] == slot_a               # the same slot ...
+    assert not graph.holds(eng._occupants([type("E", (), {"slot": slot_a})()]))   # ... but not the same request
+    replays = eng.graph_replays
+    out = eng.step([("b", [b[20]], [0])])
+    assert eng.graph_replays == replays + 1             # refilled in full and replayed
+    want = H.plain_logits(folder, b)[0][20]
+    assert (out.logits[0].double() - want).abs().max().item() <= 2e-5 * max(1.0, want.abs().max().item())
+    # the buffer's block-table line is b's now
+    (t_off, (rows, width)), = [graph.table_at[g] for g in graph.table_at][:1]
+    line = graph.host.numpy()[t_off:t_off + width]
+    table = next(iter(eng.cache.groups.values())).tables[slot_a]
+    assert list(line[:len(table)]) == table
+
+
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("D", "bfloat16")])
+@pytest.mark.parametrize("seed", [21, 22])
+def test_mixed_schedules_through_step_buffers(name, dtype, seed):
+    """Random mixed schedules with exactly as many slots as live requests: requests end, others take their slots and
+    pages, and decode steps of the same shape keep coming."""
+    import random
+    rng = random.Random(seed)
+    vocab = H.TINY[name]["cfg"].vocab_size
+    lengths = [rng.choice((3, 17, 33, 40, 64, 65, 80)) for _ in range(7)]
+    reqs = {f"r{i}": H.random_ids(vocab, n, seed * 100 + i) for i, n in enumerate(lengths)}
+    live = rng.randint(1, 3)
+    steps, peak = H.mixed_trace(reqs, max_live=live, seed=seed, prompt_frac=0.3)
+    folder, eng = engine_for(name, dtype, max_tokens=peak, max_requests=live)
+    main, _ = H.run_trace(eng, steps, heads=False)
+    assert eng.graph_replays > 0
+    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()

@@ -12,9 +12,12 @@ import torch
 
 
 class TorchOps:
-    def __init__(self, device="cpu", dtype=torch.float32):
+    def __init__(self, device="cpu", dtype=torch.float32, graphs=False):
+        """graphs: let the engine keep steps in fixed buffers and "replay" them as it does with captured graphs on
+        the GPU, only that a replay here is the same calls made again: the host side of that path without a device."""
         self.device = torch.device(device)
         self.dtype = dtype
+        self.supports_graphs = self.emulates_graphs = bool(graphs)
 
     def empty(self, *shape, dtype=None):
         return torch.zeros(*shape, dtype=dtype or self.dtype, device=self.device)

@@ -72,8 +72,15 @@ class Engine:
         self.page_size = page_size
         self.cache = CacheManager(self.model.cache_needs(), page_size, n_pages, max_requests, self.dtype, self.device)
         self.requests: Dict[Hashable, Tuple[int, int]] = {}      # id -> (slot, positions fed)
+        # a slot is handed to request after request; what a captured step keeps about "the requests it holds" must
+        # change when a slot changes hands, so every admission gets a number and a slot remembers its occupant's
+        self._admissions = 0
+        self._slot_admission: Dict[int, int] = {}
         # decode steps are replayed from captured graphs where the kernels allow it
         self.use_graphs = bool(use_graphs) and bool(getattr(ops, "supports_graphs", False)) and self.model.graph_safe
+        # an operations object without a device to capture on (a test's stand-in) may ask for the same host logic
+        # with plain launches in place of replays
+        self._capture_graphs = not getattr(ops, "emulates_graphs", False)
         self.graph_table_pages = 64          # block-table widths are rounded up to this many pages
         self._graphs: "OrderedDict[Tuple[int, int], object]" = OrderedDict()   # least recently used first
         self.max_graphs = 32                 # each holds its step's activations; the oldest goes when there are more
@@ -84,11 +91,18 @@ class Engine:
     def open(self, rid: Hashable) -> None:
         if rid in self.requests:
             raise ValueError(f"request {rid!r} is already live")
-        self.requests[rid] = (self.cache.open_request(), 0)
+        slot = self.cache.open_request()
+        self._admissions += 1
+        self._slot_admission[slot] = self._admissions
+        self.requests[rid] = (slot, 0)
 
     def close(self, rid: Hashable) -> None:
         slot, _ = self.requests.pop(rid)
+        self._slot_admission.pop(slot, None)
         self.cache.close_request(slot)
+
+    def _occupants(self, batch_entries):
+        return tuple((e.slot, self._slot_admission[e.slot]) for e in batch_entries)
 
     def reserve(self, rid: Hashable, n_tokens: int) -> None:
         """Take now every page that `rid` needs to hold `n_tokens` positions (opening it if it is not live), the way
@@ -182,31 +196,55 @@ class Engine:
                                         self.device, self.spec.max_context, getattr(self.ops, "plan_rows", None))
             outs = self.model.forward(step, self.cache)
         n = sum(len(e.want) for e in batch_entries)
-        vocab = self.spec.vocab_size
-        if logits is not None:
-            pass
-        elif n:
-            logits = self.model.logits(outs[0].hidden, step.stages[0].want_index, n)
-        else:
-            logits = torch.empty(0, vocab, dtype=torch.float32, device=self.device)
         head_logits = head_valid = None
-        if heads and len(outs) > 1:
-            head_logits, head_valid = [], []
-            for o in outs[1:]:
-                valid = o.batch.want_valid
-                if n and o.batch.n_rows and any(valid):
-                    idx = torch.clamp(o.batch.want_index[:n], min=0)
-                    lg = self.model.logits(o.hidden, idx, n)
-                    lg[~torch.tensor(valid, device=self.device)] = float("nan")
-                else:
-                    lg = torch.full((n, vocab), float("nan"), dtype=torch.float32, device=self.device)
-                head_logits.append(lg)
-                head_valid.append(list(valid))
+        if logits is None:
+            if heads and len(outs) > 1:
+                logits, head_logits, head_valid = self._all_logits(outs, n)
+            else:
+                logits = self.logits_of(outs, step, n)
         for rid, toks, _ in entries:
             slot, fed = self.requests[rid]
             self.requests[rid] = (slot, fed + len(toks))
             self.cache.release_behind(slot, fed + len(toks), self.model.max_lag)
         return StepOutput(logits, head_logits, head_valid)
+
+    def _sync(self):
+        if torch.device(self.device).type == "cuda":
+            torch.cuda.synchronize(self.device)
+
+    def logits_of(self, outs, step, n):
+        """32-bit logits [n, vocab] of the first stage's wanted rows."""
+        if n:
+            return self.model.logits(outs[0].hidden, step.stages[0].want_index, n)
+        return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
+
+    def _all_logits(self, outs, n):
+        """Logits of every stage at the wanted places from one product with the output table, which all stages share
+        (reference main_models_new.py:225-226): the table is read once however many stages there are. Rows that a
+        prediction stage does not have yet come back as NaN."""
+        vocab, S = self.spec.vocab_size, len(outs)
+        if n == 0:
+            e = torch.empty(0, vocab, dtype=torch.float32, device=self.device)
+            return e, [e.clone() for _ in outs[1:]], [[] for _ in outs[1:]]
+        rows = self.ops.empty(S * n, self.spec.d_model)
+        valid = []
+        for j, o in enumerate(outs):
+            v = [True] * n if j == 0 else list(o.batch.want_valid)
+            part = rows[j * n:(j + 1) * n]
+            if o.batch.n_rows and any(v):
+                idx = o.batch.want_index[:n] if j == 0 else torch.clamp(o.batch.want_index[:n], min=0)
+                self.ops.gather_rows(o.hidden, o.hidden, idx, out=part)
+            else:
+                part.zero_()
+            valid.append(v)
+        lg = self.ops.linear(rows, self.model.shared["lm_head"], out_dtype=torch.float32).view(S, n, vocab)
+        head_logits = []
+        for j in range(1, S):
+            h = lg[j]
+            if not all(valid[j]):
+                h[~torch.tensor(valid[j], device=self.device)] = float("nan")
+            head_logits.append(h)
+        return lg[0], head_logits, valid[1:]
 
     def _repeated_step(self, batch_entries):
         """Any other step whose shape has come before: the same requests' row counts, the same places wanted, the
@@ -229,9 +267,9 @@ class Engine:
             if seen < 2:
                 return None, plan
             if len(self._graphs) >= self.max_graphs:
-                torch.cuda.synchronize(self.device)
+                self._sync()
                 self._graphs.popitem(last=False)
-            graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size)
+            graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size, capture=self._capture_graphs)
         else:
             self._graphs.move_to_end(key)
         self.graph_replays += 1
@@ -246,7 +284,8 @@ class Engine:
         graph = self._graphs.get(key)
         if graph is not None:
             self._graphs.move_to_end(key)
-        if graph is not None and graph.slots == tuple(e.slot for e in batch_entries):
+        occupants = self._occupants(batch_entries)
+        if graph is not None and graph.holds(occupants):
             for e in batch_entries:
                 if e.start + 1 > self.spec.max_context:
                     raise ValueError(f"request in slot {e.slot} would pass the model's context of {self.spec.max_context}")
@@ -266,8 +305,9 @@ class Engine:
                 outs = self.model.forward(step, self.cache)
                 return self.model.logits(outs[0].hidden, step.stages[0].want_index, len(batch_entries))
             if len(self._graphs) >= self.max_graphs:
-                torch.cuda.synchronize(self.device)          # no replay of the graph to be dropped is still running
+                self._sync()          # no replay of the graph to be dropped is still running
                 self._graphs.popitem(last=False)
-            graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size)
+            graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size, occupants,
+                                                    capture=self._capture_graphs)
         self.graph_replays += 1
-        return graph.run(plan)
+        return graph.run(plan, occupants)

@@ -18,28 +18,48 @@ import torch
 from .batch import StepPlan, materialize
 
 
+class _NoEvent:
+    """Stands in for a device event where copies are synchronous (a host-only run)."""
+
+    def record(self):
+        pass
+
+    def synchronize(self):
+        pass
+
+
 class DecodeGraph:
-    def __init__(self, engine, plan: StepPlan, kv_capacity: int):
+    """One captured step: a fixed buffer of the step's integer arrays, and the graph that runs on it.
+
+    occupants: for every entry of the plan something that names the request itself and not merely its slot
+    (the engine passes (slot, admission number)); the quick update below is only right while the buffer's
+    lines belong to the very same requests.
+    capture=False records nothing: a replay then runs the same calls again on the same buffers. That is how an
+    operations object without a device (a test's stand-in) exercises this file's host logic.
+    """
+
+    def __init__(self, engine, plan: StepPlan, kv_capacity: int, occupants=None, capture: bool = True):
         self.layout = plan.layout()
+        self.engine = engine
+        self.capture = capture
         dev = engine.device
-        self.host = torch.zeros(max(plan.packer.total, 4), dtype=torch.int32, pin_memory=True)
+        on_gpu = torch.device(dev).type == "cuda"
+        self.host = torch.zeros(max(plan.packer.total, 4), dtype=torch.int32, pin_memory=on_gpu)
         self.dev = torch.zeros(max(plan.packer.total, 4), dtype=torch.int32, device=dev)
-        self.copied = torch.cuda.Event()
+        self.copied = torch.cuda.Event() if on_gpu else _NoEvent()
         self.step = materialize(plan, dev, self.host, self.dev)
         for st in self.step.stages:          # later steps of the shape may see more keys than this one
             st.max_kv_len = kv_capacity
-        n = self.step.n_wanted
-        self.graph = torch.cuda.CUDAGraph()
-        torch.cuda.synchronize(dev)
-        with torch.cuda.graph(self.graph):
-            outs = engine.model.forward(self.step, engine.cache)
-            if n:
-                self.logits = engine.model.logits(outs[0].hidden, self.step.stages[0].want_index, n)
-            else:
-                self.logits = torch.empty(0, engine.spec.vocab_size, dtype=torch.float32, device=dev)
+        self.graph = None
+        if capture:
+            self.graph = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize(dev)
+            with torch.cuda.graph(self.graph):
+                self._launch()
         self.copied.record()
         # what the quick update needs: which requests, in which order, the buffer holds, and where their arrays lie
         self.slots = tuple(e.slot for e in plan.entries)
+        self.occupants = tuple(occupants) if occupants is not None else None
         self.cache = engine.cache
         self.page_size = engine.page_size
         off = lambda i: plan.packer.offsets[i][0]
@@ -48,6 +68,21 @@ class DecodeGraph:
                               ws={g: off(i) for g, i in pl["ws"].items()}) for pl in plan.plans]
         self.pages_held = {g: np.array([len(engine.cache.groups[g].tables[s]) for s in self.slots])
                            for g in self.table_at}
+
+    def _launch(self):
+        engine, n = self.engine, self.step.n_wanted
+        outs = engine.model.forward(self.step, engine.cache)
+        self.logits = engine.logits_of(outs, self.step, n)
+
+    def _replay(self):
+        if self.graph is not None:
+            self.graph.replay()
+        else:
+            self._launch()
+
+    def holds(self, occupants) -> bool:
+        """Whether the buffer's lines are those of exactly these requests, in this order."""
+        return self.occupants is not None and self.occupants == tuple(occupants)
 
     def run_same_requests(self, entries) -> torch.Tensor:
         """The next step of the very requests whose arrays the buffer already holds, in the same order: only
@@ -78,10 +113,10 @@ class DecodeGraph:
                 flat[w_off:w_off + n] = table[rows_idx, pos // ps] * ps + pos % ps
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
-        self.graph.replay()
+        self._replay()
         return self.logits
 
-    def run(self, plan: StepPlan) -> torch.Tensor:
+    def run(self, plan: StepPlan, occupants=None) -> torch.Tensor:
         if plan.layout() != self.layout:
             raise RuntimeError("this step's arrays do not have the captured layout")
         self.copied.synchronize()            # the previous copy out of the pinned buffer has finished
@@ -89,7 +124,8 @@ class DecodeGraph:
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
         self.slots = tuple(e.slot for e in plan.entries)
+        self.occupants = tuple(occupants) if occupants is not None else None
         for g in self.table_at:
             self.pages_held[g] = np.array([len(self.cache.groups[g].tables[s]) for s in self.slots])
-        self.graph.replay()
+        self._replay()
         return self.logits

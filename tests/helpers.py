@@ -28,6 +28,22 @@ TINY = {
     "D": dict(cfg=GqaMtpConfig(d_model=256, vocab_size=515, max_context=640, rope_base=10000.0, n_heads=2, n_layers=2,
                                ffn_hidden=320, group_size=2, mtp_heads=2, rms_eps=2e-8, tie_embeddings=False),
               page_size=16, gain_jitter=0.05, seed=14),
+    # the headline size's layer sizes (1536 wide, 12 query heads of 128 over 3, feed-forward 4096, two prediction
+    # heads) with 2 of its 30 layers and a small vocabulary
+    "E": dict(cfg=GqaMtpConfig(d_model=1536, vocab_size=1000, max_context=2304, rope_base=10000.0, n_heads=12,
+                               n_layers=2, ffn_hidden=4096, group_size=4, mtp_heads=2, rms_eps=2e-8,
+                               tie_embeddings=True),
+              page_size=16, gain_jitter=0.1, seed=15),
+    # the attention geometries of the two larger sizes (16 heads of 128 over 4; 32 over 8) with one layer and a
+    # narrow feed-forward
+    "F": dict(cfg=GqaMtpConfig(d_model=2048, vocab_size=900, max_context=1536, rope_base=10000.0, n_heads=16,
+                               n_layers=1, ffn_hidden=1408, group_size=4, mtp_heads=2, rms_eps=2e-8,
+                               tie_embeddings=True),
+              page_size=16, gain_jitter=0.1, seed=16),
+    "G": dict(cfg=GqaMtpConfig(d_model=4096, vocab_size=600, max_context=1024, rope_base=500000.0, n_heads=32,
+                               n_layers=1, ffn_hidden=1024, group_size=4, mtp_heads=1, rms_eps=2e-8,
+                               tie_embeddings=False),
+              page_size=16, gain_jitter=0.1, seed=17),
 }
 
 _folders: Dict[Tuple[str, str], str] = {}
@@ -139,6 +155,26 @@ def mixed_trace(reqs: Dict[str, List[int]], max_live: int = 4, seed: int = 0, pr
     return steps, peak
 
 
+def wanted_keys(steps, n_heads: int):
+    """What a trace asks for: the (id, position) of every wanted place, and for every prediction head the
+    (id, head, head position) it owes there: head i answers a wanted position p with its row p - 1 - i, once
+    that is a position at all."""
+    fed: Dict[str, int] = {}
+    main, heads = set(), set()
+    for st in steps:
+        for e in st["entries"]:
+            start = fed.get(e["id"], 0)
+            for i in e["want"]:
+                main.add((e["id"], start + i))
+                for hi in range(n_heads):
+                    if start + i - 1 - hi >= 0:
+                        heads.add((e["id"], hi, start + i - 1 - hi))
+            fed[e["id"]] = start + len(e["tokens"])
+        for rid in st["end"]:
+            fed.pop(rid, None)
+    return main, heads
+
+
 def run_trace(engine, steps, heads: bool = True):
     """Drive the engine's step function; returns {(id, position): logits} and {(id, head, head position): logits}."""
     main: Dict[Tuple[str, int], torch.Tensor] = {}
@@ -163,8 +199,17 @@ def run_trace(engine, steps, heads: bool = True):
     return main, head_out
 
 
-def compare_with_plain(folder, reqs, main, head_out, tol, n_heads):
-    """Largest absolute difference against the plain implementation, asserted below `tol`, with the place named."""
+def compare_with_plain(folder, reqs, main, head_out, tol, n_heads, steps=None):
+    """Largest absolute difference against the plain implementation, asserted below `tol`, with the place named.
+    With `steps` (the trace that was run) also: everything the trace asked for came back, and nothing else."""
+    if steps is not None:
+        want_main, want_heads = wanted_keys(steps, n_heads)
+        assert set(main) == want_main, f"main logits: missing {sorted(want_main - set(main))[:5]}, " \
+                                       f"unasked {sorted(set(main) - want_main)[:5]}"
+        assert set(head_out) == want_heads, f"head logits: missing {sorted(want_heads - set(head_out))[:5]}, " \
+                                            f"unasked {sorted(set(head_out) - want_heads)[:5]}"
+        for rid, hi, p in want_heads:
+            assert p < len(reqs[rid]) - 1 - hi
     worst = (0.0, None)
     for rid, ids in reqs.items():
         pm_main, pm_heads = plain_logits(folder, ids)
@@ -191,3 +236,19 @@ def first_wrong(folder, reqs, main, tol):
             if (rid, p) in main and not (main[(rid, p)].double() - pm_main[p]).abs().max().item() <= tol:
                 return rid, p
     return None
+
+
+SLOT_CASES = [(1, "final", None), (2, "final", None), (2, "cur", 80), (3, "cur", 96)]   # max_batch, plan, pool tokens
+
+
+def slot_pressure_workload(name: str):
+    """Five greedy requests of different prompt and output lengths, so that in a batch the newest often finishes first
+    and its successor takes its slot: (folder, prompts, sampling params, the plain model's tokens)."""
+    from tiny_inference_server_amd.sampling import SamplingParams
+    folder = model_folder(name, "float32")
+    cfg, w = pm.read_model_folder(folder)
+    lens, new = [30, 7, 12, 19, 5], [24, 5, 9, 14, 20]
+    prompts = [random_ids(cfg["vocab"], n, 190 + i) for i, n in enumerate(lens)]
+    params = [SamplingParams(max_new_tokens=k, temperature=0.0, ignore_eos=True) for k in new]
+    want = [pm.greedy_generate(p, k, w, cfg) for p, k in zip(prompts, new)]
+    return folder, prompts, params, want

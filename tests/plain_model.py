@@ -2,7 +2,7 @@
 
 Whole sequences, no cache, no batching, one function for each part, float64 by default. It shares no code
 with the engine: it reads config.json and model.safetensors itself. Each function cites the lines of the
-reference (under /root/reference) that it follows. The reference was read, not run.
+reference (main_models_new.py, server.py, ...) that it follows. The reference was read, not run.
 """
 from __future__ import annotations
 

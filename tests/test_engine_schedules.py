@@ -40,6 +40,9 @@ def scale_of(folder, reqs):
 
 CASES = [("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16"), ("C", "bfloat16"),
          ("D", "bfloat16"), ("D", "float32")]
+# the layer sizes of the headline model and the attention geometries of the two larger ones: on the GPU only (their
+# plain results alone take the CPU a while)
+BIG_CASES = [pytest.param(n, "bfloat16", "hip", marks=pytest.mark.gpu) for n in ("E", "F", "G")]
 
 
 @pytest.mark.parametrize("backend", backends())
@@ -47,8 +50,9 @@ CASES = [("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16"
 def test_whole_requests(name, dtype, backend):
     reqs = requests_for(name, [5, 17, 33, 1, 2, 70], seed=1)
     folder, eng = make_engine(name, dtype, backend, max_tokens=128)
-    main, heads = H.run_trace(eng, H.whole_trace(reqs))
-    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    steps = H.whole_trace(reqs)
+    main, heads = H.run_trace(eng, steps)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads, steps)
     eng.cache.check()
     assert eng.free_pages() == eng.total_pages()
 
@@ -58,8 +62,9 @@ def test_whole_requests(name, dtype, backend):
 def test_prefill_then_decode_one_by_one(name, dtype, backend):
     reqs = requests_for(name, [75, 40, 33], seed=2)
     folder, eng = make_engine(name, dtype, backend, max_tokens=128)
-    main, heads = H.run_trace(eng, H.tail_decode_trace(reqs, tail=32))
-    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    steps = H.tail_decode_trace(reqs, tail=32)
+    main, heads = H.run_trace(eng, steps)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads, steps)
     assert eng.free_pages() == eng.total_pages()
 
 
@@ -68,8 +73,9 @@ def test_prefill_then_decode_one_by_one(name, dtype, backend):
 def test_portions_of_changing_size(name, dtype, backend):
     reqs = requests_for(name, [97, 50], seed=3)
     folder, eng = make_engine(name, dtype, backend, max_tokens=128)
-    main, heads = H.run_trace(eng, H.portions_trace(reqs, seed=1))
-    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    steps = H.portions_trace(reqs, seed=1)
+    main, heads = H.run_trace(eng, steps)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads, steps)
     assert eng.free_pages() == eng.total_pages()
 
 
@@ -83,7 +89,7 @@ def test_mixed_batches_with_page_reuse(name, dtype, backend):
     folder, eng = make_engine(name, dtype, backend, max_tokens=peak)
     assert sum(-(-n // 64) * 64 for n in lengths) > 2 * peak
     main, heads = H.run_trace(eng, steps)
-    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads, steps)
     eng.cache.check()
     assert eng.free_pages() == eng.total_pages()
 
@@ -103,7 +109,7 @@ def test_first_tokens_and_long_decoding(name, dtype, backend):
     M = eng.config.mtp_heads
     for hi in range(M):
         assert all(("r0", hi, p) in heads for p in range(n - 1 - hi))
-    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), M)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), M, steps)
 
 
 @pytest.mark.parametrize("backend", backends())
@@ -145,7 +151,8 @@ def test_schedules_with_portions_on_the_tile_kernel(name, monkeypatch):
         folder, eng = make_engine(name, "bfloat16", "hip", max_tokens=max_tokens)
         main, heads = H.run_trace(eng, trace)
         assert planned["tiles"] > 0          # whole prompts always fill tiles; the short portions of C may not
-        H.compare_with_plain(folder, reqs, main, heads, TOL["bfloat16"] * scale_of(folder, reqs), eng.config.mtp_heads)
+        H.compare_with_plain(folder, reqs, main, heads, TOL["bfloat16"] * scale_of(folder, reqs), eng.config.mtp_heads,
+                             trace)
         eng.cache.check()
         assert eng.free_pages() == eng.total_pages()
 
@@ -165,7 +172,7 @@ def test_long_context_decoding_in_bfloat16():
         p += n
     main, _ = H.run_trace(eng, steps, heads=False)
     assert eng.graph_replays >= 100
-    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0)
+    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0, steps)
 
 
 @pytest.mark.parametrize("backend", backends())
@@ -181,7 +188,7 @@ def test_random_schedules(name, dtype, backend, seed):
     steps, peak = H.mixed_trace(reqs, max_live=rng.randint(1, 4), seed=seed, prompt_frac=rng.choice((0.0, 0.3, 0.7, 1.0)))
     folder, eng = make_engine(name, dtype, backend, max_tokens=peak)
     main, heads = H.run_trace(eng, steps)
-    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads, steps)
     eng.cache.check()
     assert eng.free_pages() == eng.total_pages()
 
@@ -198,4 +205,53 @@ def test_what_a_page_held_before_never_reaches_a_result(name, dtype, backend):
     for g in eng.cache.groups.values():
         g.storage.fill_(float("nan"))
     main, heads = H.run_trace(eng, steps)
-    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads, steps)
+
+
+@pytest.mark.parametrize("name,dtype,backend", BIG_CASES)
+def test_schedule_families_at_model_geometries(name, dtype, backend):
+    """Whole prompts, prompt then decoding one by one, portions of changing size, and mixed batches on few pages, at
+    the headline model's layer sizes (E: 12 query heads of 128 over 3 key/value heads) and at the attention
+    geometries of the larger sizes (F: 16 over 4, G: 32 over 8): the matrix-core kernels with a group of four, several
+    key/value heads, the few-row products at these widths. Nothing is patched; the planner chooses as it does in use."""
+    reqs = requests_for(name, [5, 33, 70, 90, 47, 18], seed=21)
+    mixed, peak = H.mixed_trace(reqs, max_live=4, seed=22)
+    for steps, max_tokens in ((H.whole_trace(reqs), 128), (H.tail_decode_trace(reqs, tail=32), 128),
+                              (H.portions_trace(reqs, seed=3), 128), (mixed, peak)):
+        folder, eng = make_engine(name, dtype, backend, max_tokens=max_tokens)
+        main, heads = H.run_trace(eng, steps)
+        H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), eng.config.mtp_heads, steps)
+        eng.cache.check()
+        assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,cut", [("E", (1600, 448)), ("F", (1296, 200)), ("G", (900, 100))])
+def test_long_prompt_cut_in_two_at_model_geometries(name, cut, monkeypatch):
+    """A long prompt in two portions, then a few tokens one by one. The first portion is long enough for the planner
+    to give it to the workgroup (tile) attention kernel at its real thresholds and to the sixteen-row rotary kernel;
+    the second runs behind it over the paged context, its key ranges split and merged; the prediction heads run
+    their shifted rows. Every position's main and head logits are compared with the plain implementation."""
+    from tiny_inference_server_amd.ops import hip_ops
+    planned = {"tiles": 0, "items": 0}
+    plan = hip_ops.attention_items
+
+    def counting(*args, **kw):
+        out = plan(*args, **kw)
+        planned["items"] += len(out[1])
+        planned["tiles"] += len(out[2])
+        return out
+    monkeypatch.setattr(hip_ops, "attention_items", counting)
+    n = sum(cut) + 4
+    reqs = requests_for(name, [n], seed=23)
+    ids = reqs["r0"]
+    folder, eng = make_engine(name, "bfloat16", "hip", max_tokens=-(-n // 64) * 64)
+    steps, p = [], 0
+    for k in list(cut) + [1] * 4:
+        steps.append({"step": len(steps), "entries": [{"id": "r0", "tokens": ids[p:p + k], "want": list(range(k))}],
+                      "end": ["r0"] if p + k == n else []})
+        p += k
+    main, heads = H.run_trace(eng, steps)
+    assert planned["tiles"] > 0 and planned["items"] > 0
+    H.compare_with_plain(folder, reqs, main, heads, TOL["bfloat16"] * scale_of(folder, reqs), eng.config.mtp_heads, steps)
+    assert eng.free_pages() == eng.total_pages()

@@ -49,6 +49,36 @@ def test_bfloat16_generation_follows_the_plain_choice_where_it_is_clear():
             ids.append(t)
 
 
+def test_bfloat16_scheduler_with_heads_and_preemption():
+    """The scheduler on the GPU in bfloat16 with the prediction heads run at every step, as many slots as requests,
+    a pool that forces preemption under plan "cur", and prompts cut by a small token budget (the reference's own
+    model-level check of its scheduler: test_server.py:66-118). Tokens are compared with the plain model's choice
+    wherever that choice is clear (bfloat16 may flip an arg-max between two close logits)."""
+    folder = H.model_folder("D", "bfloat16")
+    cfg, w = pm.read_model_folder(folder)
+    lens, new = [30, 12, 21, 9, 17], [20, 6, 12, 16, 8]
+    prompts = [H.random_ids(cfg["vocab"], n, 140 + i) for i, n in enumerate(lens)]
+    params = [SamplingParams(max_new_tokens=k, temperature=0.0, ignore_eos=True) for k in new]
+    got, s = generate(folder, prompts, params=params, dtype="bfloat16", max_batch=3, token_budget=24, plan="cur",
+                      pool_tokens=96, run_heads=True, return_scheduler=True)
+    assert s.preempts > 0 and s.engine.graph_replays > 0
+    assert len(s.engine.model.spec.stages) == 3          # the heads did run
+    checked = 0
+    for p, g, k in zip(prompts, got, new):
+        assert len(g) == k
+        ids = list(p)
+        for t in g:
+            lg = pm.logits_of(pm.trunk_hidden(ids, w, cfg)[-1:], w, cfg)[0]
+            top2 = torch.topk(lg, 2).values
+            if (top2[0] - top2[1]).item() > 0.1:
+                assert t == int(lg.argmax())
+                checked += 1
+            ids.append(t)
+    assert checked >= sum(new) // 2
+    s.engine.cache.check()
+    assert s.engine.free_pages() == s.engine.total_pages()
+
+
 def test_temperature_sampling_with_seeded_streams():
     """Tiny B's workload: temperature 0.8, seed 0, mixed chunked prefill and decode; token by token the draw is the
     plain rule's (server.py:22-50) on the plain logits with the request's own uniform number."""

@@ -35,6 +35,7 @@ def test_graph_replays_match_eager_steps(name):
                 torch.cuda.synchronize()
     assert engines[True].graph_replays >= 20 and engines[False].graph_replays == 0
     tol = 2e-2 * max(1.0, max(H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values()))
+    assert set(got[True]) == set(got[False]) == {(r, p) for r, ids in reqs.items() for p in range(prompt, min(47, len(ids)))}
     H.compare_with_plain(folder, reqs, got[True], {}, tol, 0)
     H.compare_with_plain(folder, reqs, got[False], {}, tol, 0)
     # two bfloat16 runs that are each within tol of the plain result are within 2 tol of each other; the graph
@@ -64,6 +65,7 @@ def test_graph_survives_changing_batches(max_graphs):
         for k, r in enumerate(live):
             main[(r, fed[r])] = lg[k]
             fed[r] += 1
+    assert set(main) == {(r, p) for r, ids in reqs.items() for p in range(10, len(ids))}
     assert min(3, max_graphs) <= len(eng._graphs) <= max_graphs and eng.graph_replays >= 30
     H.compare_with_plain(folder, reqs, main, {}, 2e-2 * max(1.0, max(
         H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values())), 0)
@@ -100,3 +102,42 @@ def test_repeated_prompt_steps_are_replayed(name):
     assert eng.graph_replays >= 4
     eng.cache.check()
     assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("D", "bfloat16"), ("C", "bfloat16")])
+def test_requests_follow_each_other_through_one_slot(name, dtype):
+    """As many slots as live requests: one. Every request takes over its predecessor's slot at the same place in the
+    batch; the second holds fewer pages than the first did, the third more. A captured step must run on the new
+    owner's block table (finished requests leave and queued ones take their places: reference server.py:286-292)."""
+    from test_step_buffers import one_after_the_other
+    folder = H.model_folder(name, "float32" if dtype == "float32" else "bfloat16")
+    vocab = H.TINY[name]["cfg"].vocab_size
+    reqs = {f"s{i}": H.random_ids(vocab, n, 90 + i) for i, n in enumerate([70, 40, 75, 41])}
+    eng = Engine(folder, dtype=dtype, page_size=H.TINY[name]["page_size"], max_tokens=256, max_requests=1)
+    assert eng.use_graphs
+    steps = one_after_the_other(reqs, 9)
+    main, _ = H.run_trace(eng, steps, heads=False)
+    assert eng.graph_replays > 100
+    tol = (2e-5 if dtype == "float32" else 2e-2) * max(1.0, max(
+        H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values()))
+    H.compare_with_plain(folder, reqs, main, {}, tol, 0, steps)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("max_batch,plan,pool", H.SLOT_CASES)
+def test_generation_with_as_many_slots_as_requests(name, max_batch, plan, pool):
+    """generate() gives the engine exactly max_batch slots. Requests of different lengths, the newest of a batch
+    finishing first, its successor taking its slot; with plan "cur" on a small pool requests are preempted and
+    admitted again into slots others have used meanwhile. Greedy tokens in 32-bit equal the plain model's."""
+    from tiny_inference_server_amd.engine.generate import generate
+    folder, prompts, params, want = H.slot_pressure_workload(name)
+    got, s = generate(folder, prompts, params=params, dtype="float32", tokens_per_block=H.TINY[name]["page_size"],
+                      max_batch=max_batch, token_budget=16, plan=plan, pool_tokens=pool, return_scheduler=True)
+    assert s.engine.cache.max_requests == max_batch
+    assert s.engine.graph_replays > 0
+    assert (s.preempts > 0) == (pool is not None)
+    assert got == want
+    s.engine.cache.check()
+    assert s.engine.free_pages() == s.engine.total_pages()

@@ -46,11 +46,11 @@ def test_a_slot_that_changes_hands_gets_its_new_owners_pages(name, dtype):
     reqs = {f"s{i}": H.random_ids(vocab, n, 90 + i) for i, n in enumerate([70, 40, 75, 41])}
     folder, eng = engine_for(name, dtype, max_tokens=256, max_requests=1)
     assert eng.use_graphs
-    main, _ = H.run_trace(eng, one_after_the_other(reqs, 9), heads=False)
+    steps = one_after_the_other(reqs, 9)
+    main, _ = H.run_trace(eng, steps, heads=False)
     assert eng.graph_replays > 100
-    wanted = {(rid, p) for rid, ids in reqs.items() for p in range(8, len(ids))}
-    assert set(main) == wanted
-    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0)
+    assert set(main) == {(rid, p) for rid, ids in reqs.items() for p in range(8, len(ids))}
+    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0, steps)
     eng.cache.check()
     assert eng.free_pages() == eng.total_pages()
 
@@ -99,6 +99,25 @@ def test_mixed_schedules_through_step_buffers(name, dtype, seed):
     folder, eng = engine_for(name, dtype, max_tokens=peak, max_requests=live)
     main, _ = H.run_trace(eng, steps, heads=False)
     assert eng.graph_replays > 0
-    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0)
+    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0, steps)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("max_batch,plan,pool", H.SLOT_CASES)
+def test_generation_with_as_many_slots_as_requests(name, max_batch, plan, pool):
+    """The scheduler above an engine that has exactly max_batch slots: finished and preempted requests hand their
+    slots on, decode steps of the same shape keep coming, and the greedy tokens are the plain model's."""
+    from tiny_inference_server_amd.engine.generate import generate
+    folder, prompts, params, want = H.slot_pressure_workload(name)
+    ps = H.TINY[name]["page_size"]
+    longest = max(len(p) + sp.max_new_tokens for p, sp in zip(prompts, params))
+    eng = Engine(folder, dtype="float32", page_size=ps, max_requests=max_batch, ops=TorchOps(graphs=True),
+                 max_tokens=pool if pool is not None else max_batch * (-(-longest // ps) * ps), run_heads=False)
+    got, s = generate(eng, prompts, params=params, max_batch=max_batch, token_budget=16, plan=plan, return_scheduler=True)
+    assert eng.graph_replays > 0
+    assert (s.preempts > 0) == (pool is not None)
+    assert got == want
     eng.cache.check()
     assert eng.free_pages() == eng.total_pages()

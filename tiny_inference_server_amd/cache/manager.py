@@ -94,8 +94,8 @@ class PageGroup:
         self.storage = None
         if allocate:
             # [plane][page][key or value][kv head][slot in page][head size]; within a page and head the values
-            # lie transposed, [head size][slot]. Zeroed once: kernels that multiply masked slots by an exact 0
-            # need every value ever found in the pool to be finite (the reference zeroes too: block_table.py:40)
+            # lie transposed, [head size][slot]. Zeroed once, as the reference does (block_table.py:40), though no
+            # kernel needs it: slots that a row may not see are read, but replaced before any arithmetic
             self.storage = torch.zeros((len(spec.keys), n_pages, 2, spec.n_kv_heads, page_size, spec.head_dim),
                                        dtype=dtype, device=device)
 

@@ -283,17 +283,11 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
   }
 }
 
-// A hook for tuning runs: forces (waves, U, R) for every launch of this process; zeros give the choice back.
-static int g_force_waves = 0, g_force_u = 0, g_force_r = 0;
+// (both can be set from outside: the kernel tests make small matrices take the wide path)
 static int g_wide_tiles = 256;   // from this many 32-column workgroups on (one a compute unit), a workgroup takes two column tiles
 static int g_wide_max_blocks = 2;   // with up to two blocks of 16 rows (four blocks measured no gain over the library)
 TIS_EXPORT void tis_gemm_skinny_wide_tiles(int n_workgroups) { g_wide_tiles = n_workgroups; }
 TIS_EXPORT void tis_gemm_skinny_wide_max_blocks(int n) { g_wide_max_blocks = n; }
-TIS_EXPORT void tis_gemm_skinny_force_config(int waves, int u, int r) {
-  g_force_waves = waves;
-  g_force_u = u;
-  g_force_r = r;
-}
 
 
 template <bool NORM, int EPI, typename TO>
@@ -303,7 +297,6 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
   // rows allow it (measured at N = 1536: 6.2 instead of 8.2 us for K = 4096, 4.1 instead of 4.8 us for K = 1536;
   // at N = 2304 with the norm in front the wider tile stays ahead, and a quarter tile never beat the half)
   int r = (M <= 8 && (N + 15) / 16 <= 128) ? 2 : 1;
-  if (g_force_r) r = g_force_r;
   if (r != 1 && r != 2) return tis_fail("gemm_skinny: %d chunks a step; 1 or 2 are built", r);
   if (r == 2 && M > 8) return tis_fail("gemm_skinny: %d rows do not fit 8 columns a workgroup", M);
   const int mb = M <= 16 ? 1 : M <= 32 ? 2 : 4;
@@ -317,7 +310,6 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
     waves = 4;
     u = (steps % 3 == 0 && steps % 4 != 0) || steps == 12 ? 3 : 4;
   }
-  if (g_force_waves) { waves = g_force_waves; u = g_force_u; }
   if (mb > 1 && waves != 8) { waves = 8; u = 4; }   // several row blocks are built for eight waves only
   // two column tiles a workgroup where the matrix is wide enough to fill the chip with half as many workgroups:
   // the activations, the gains and the norm's arithmetic are then shared by twice as many weights (the gate-up

@@ -2,8 +2,9 @@
 
 Every method checks on the host that shapes, dtypes and strides are what the kernel and its grid assume,
 then launches on torch's current stream. There is no CPU path: without a GPU or without the compiled
-libraries construction fails. Matrix products in bfloat16 go to the library behind torch.matmul, as the
-reference's do (main_models_new.py:19-20); in 32-bit they go to the plain multiply-add kernel so that no
+libraries construction fails. Matrix products in bfloat16 of a few rows go to the fused few-row kernel
+(csrc/gemm_skinny.hip), those of many rows to hipBLASLt through csrc/gemm_library.hip, as the reference's go to
+a library (main_models_new.py:19-20); in 32-bit they go to the plain multiply-add kernel so that no
 reduced-precision matrix mode can take part.
 """
 from __future__ import annotations

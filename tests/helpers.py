@@ -28,22 +28,26 @@ TINY = {
     "D": dict(cfg=GqaMtpConfig(d_model=256, vocab_size=515, max_context=640, rope_base=10000.0, n_heads=2, n_layers=2,
                                ffn_hidden=320, group_size=2, mtp_heads=2, rms_eps=2e-8, tie_embeddings=False),
               page_size=16, gain_jitter=0.05, seed=14),
+    # Matrices of the wide configurations are drawn with the standard deviation the sizes are specified with (0.02;
+    # with 0.05 every product of 1536 inputs doubles the stream's scale and with it bfloat16's rounding error), and
+    # their query projections are then multiplied by `sharpen`, so that attention weights are far from uniform and a
+    # wrong key, mask or page moves the result.
     # the headline size's layer sizes (1536 wide, 12 query heads of 128 over 3, feed-forward 4096, two prediction
     # heads) with 2 of its 30 layers and a small vocabulary
     "E": dict(cfg=GqaMtpConfig(d_model=1536, vocab_size=1000, max_context=2304, rope_base=10000.0, n_heads=12,
                                n_layers=2, ffn_hidden=4096, group_size=4, mtp_heads=2, rms_eps=2e-8,
                                tie_embeddings=True),
-              page_size=16, gain_jitter=0.1, seed=15),
+              page_size=16, gain_jitter=0.1, seed=15, std=0.02, sharpen=2.0),
     # the attention geometries of the two larger sizes (16 heads of 128 over 4; 32 over 8) with one layer and a
     # narrow feed-forward
     "F": dict(cfg=GqaMtpConfig(d_model=2048, vocab_size=900, max_context=1536, rope_base=10000.0, n_heads=16,
                                n_layers=1, ffn_hidden=1408, group_size=4, mtp_heads=2, rms_eps=2e-8,
                                tie_embeddings=True),
-              page_size=16, gain_jitter=0.1, seed=16),
+              page_size=16, gain_jitter=0.1, seed=16, std=0.02, sharpen=2.0),
     "G": dict(cfg=GqaMtpConfig(d_model=4096, vocab_size=600, max_context=1024, rope_base=500000.0, n_heads=32,
                                n_layers=1, ffn_hidden=1024, group_size=4, mtp_heads=1, rms_eps=2e-8,
                                tie_embeddings=False),
-              page_size=16, gain_jitter=0.1, seed=17),
+              page_size=16, gain_jitter=0.1, seed=17, std=0.02, sharpen=2.0),
 }
 
 _folders: Dict[Tuple[str, str], str] = {}
@@ -59,7 +63,15 @@ def model_folder(name: str, storage: str = "bfloat16") -> str:
             _tmp = tempfile.TemporaryDirectory(prefix="tis_amd_models_")
         t = TINY[name]
         _folders[key] = write_random_model(t["cfg"], t["seed"], os.path.join(_tmp.name, f"{name}_{storage}"),
-                                           std=0.05, gain_jitter=t["gain_jitter"], dtype=storage)
+                                           std=t.get("std", 0.05), gain_jitter=t["gain_jitter"], dtype=storage)
+        if t.get("sharpen"):
+            from safetensors.torch import load_file, save_file
+            path = os.path.join(_folders[key], "model.safetensors")
+            tensors = load_file(path)
+            for n in tensors:
+                if n.endswith("att.q_proj.weight"):
+                    tensors[n] = (tensors[n].float() * t["sharpen"]).to(tensors[n].dtype)
+            save_file(tensors, path)
     return _folders[key]
 
 

@@ -1,0 +1,111 @@
+"""The attention entry point that allocates nothing, called through ctypes, against the one that takes a workspace.
+
+tis_attention_mfma_static keeps the partial results of split key ranges in an array that the library holds on the
+device; tis_attention_mfma gets the same buffers from its caller. Both launch the same kernels with the same split
+counts, so their outputs must be equal bit for bit: on two calls in a row, the second smaller than the first (what
+the first call left in the array must not matter), then on a call with rows of a prompt portion beside decoded tokens
+(per-row split counts). A call whose partial results do not fit the array is refused before anything is launched.
+"""
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+HD, NH, KVH, PAGE = 128, 12, 3, 16
+
+
+def _ptr(t):
+    return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
+
+
+def _case(seed, rows_spec):
+    """rows_spec: (first position, rows) per request. Returns the kernel's inputs on the GPU."""
+    g = torch.Generator().manual_seed(seed)
+    dev = "cuda:0"
+    n_seqs = len(rows_spec)
+    width = max(-(-(p0 + n) // PAGE) for p0, n in rows_spec)
+    n_pages = n_seqs * width + 8          # every request's pages are its own, scattered over the pool
+    plane = (torch.randn(n_pages, 2, KVH, PAGE, HD, generator=g) * 0.5).to(torch.bfloat16).to(dev)
+    perm = torch.randperm(n_pages, generator=g)[:n_seqs * width].to(torch.int32).view(n_seqs, width)
+    row_seq, positions, items = [], [], []
+    for k, (p0, n) in enumerate(rows_spec):
+        first = len(row_seq)
+        row_seq += [k] * n
+        positions += list(range(p0, p0 + n))
+        per = max(1, 32 // (NH // KVH))                 # rows of one item with two column blocks
+        for r in range(0, n, per):
+            items.append((first + r, min(per, n - r)))
+    n = len(row_seq)
+    q = (torch.randn(n, NH * HD, generator=g)).to(torch.bfloat16).to(dev)
+    as_dev = lambda a: torch.tensor(a, dtype=torch.int32).to(dev)
+    return dict(q=q, plane=plane, tables=perm.to(dev).contiguous(), row_seq=as_dev(row_seq), positions=as_dev(positions),
+                items=as_dev(items).contiguous(), n_items=len(items), n=n,
+                single=all(c == 1 for _, c in rows_spec))
+
+
+def _run_both(lib, static_fn, c, n_splits, min_steps):
+    dev = c["q"].device
+    stream = c_void_p(torch.cuda.current_stream().cuda_stream)
+    items = None if c["single"] else c["items"]
+    nb = 1 if c["single"] else 2
+    n = c["n"]
+    scale = HD ** -0.5
+    out_a = torch.zeros(n, NH * HD, dtype=torch.bfloat16, device=dev)
+    out_b = torch.full((n, NH * HD), 7.0, dtype=torch.bfloat16, device=dev)
+    work = torch.full((n * NH * n_splits * (HD + 2) + n,), float("nan"), dtype=torch.float32, device=dev)
+    part_ml = work[n * NH * n_splits * HD:]
+    row_splits = work[n * NH * n_splits * (HD + 2):]
+    lib.tis_attention_mfma(_ptr(c["q"]), c["q"].stride(0), _ptr(c["plane"]), _ptr(c["tables"]), c["tables"].stride(0),
+                           _ptr(c["row_seq"]), _ptr(c["positions"]), _ptr(items), c["n_items"], nb, _ptr(None), 0,
+                           _ptr(out_a), out_a.stride(0), _ptr(work), _ptr(part_ml), n, NH, KVH, HD, PAGE, 0, scale,
+                           n_splits, min_steps, 1, 1 << 20, _ptr(row_splits), stream)
+    rc = static_fn(_ptr(c["q"]), c["q"].stride(0), _ptr(c["plane"]), _ptr(c["tables"]), c["tables"].stride(0),
+                   _ptr(c["row_seq"]), _ptr(c["positions"]), _ptr(items), c["n_items"], nb, _ptr(None), 0,
+                   _ptr(out_b), out_b.stride(0), n, NH, KVH, HD, PAGE, 0, scale, n_splits, min_steps, 1, 1 << 20, stream)
+    assert rc == 0, lib.cdll.tis_attention_mfma_last_error()
+    torch.cuda.synchronize()
+    return out_a, out_b
+
+
+def test_static_workspace_entry_point_matches_the_one_with_a_workspace():
+    from tiny_inference_server_amd.ops import hip_ops
+    lib = hip_ops.library(f"attention_mfma@{HD}")
+    fn = lib.cdll.tis_attention_mfma_static
+    fn.restype = c_int
+    fn.argtypes = [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                   c_int, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                   c_int, c_void_p]
+    lib.cdll.tis_attention_mfma_static_floats.restype = c_long
+    capacity = lib.cdll.tis_attention_mfma_static_floats()
+    assert capacity == 2 << 20
+    lib.cdll.tis_attention_mfma_last_error.restype = ctypes.c_char_p
+    # two calls in a row: sixteen decoded tokens with their keys in four splits, then five in three
+    first = _case(1, [(100 + 53 * i, 1) for i in range(16)])
+    a, b = _run_both(lib, fn, first, n_splits=4, min_steps=0)
+    assert torch.isfinite(a.float()).all() and torch.equal(a, b)
+    second = _case(2, [(700, 1), (33, 1), (515, 1), (128, 1), (257, 1)])
+    a, b = _run_both(lib, fn, second, n_splits=3, min_steps=0)
+    assert torch.isfinite(a.float()).all() and torch.equal(a, b)
+    # rows of a portion beside decoded tokens: items choose their own number of splits, the merge reads it per row
+    mixed = _case(3, [(300, 40), (900, 1), (5, 1), (0, 20)])
+    a, b = _run_both(lib, fn, mixed, n_splits=6, min_steps=2)
+    assert torch.isfinite(a.float()).all() and torch.equal(a, b)
+    # too large for the array: refused with a message, nothing launched, the output untouched
+    big = _case(4, [(1000, 1)] * 64)
+    n = big["n"]
+    splits = capacity // (n * NH * (HD + 2)) + 1
+    out = torch.full((n, NH * HD), 7.0, dtype=torch.bfloat16, device="cuda:0")
+    rc = fn(_ptr(big["q"]), big["q"].stride(0), _ptr(big["plane"]), _ptr(big["tables"]), big["tables"].stride(0),
+            _ptr(big["row_seq"]), _ptr(big["positions"]), _ptr(None), big["n_items"], 1, _ptr(None), 0, _ptr(out),
+            out.stride(0), n, NH, KVH, HD, PAGE, 0, HD ** -0.5, splits, 0, 1, 1 << 20,
+            c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert rc != 0 and b"workspace holds" in lib.cdll.tis_attention_mfma_last_error()
+    assert (out == 7.0).all()
+    # and the first case once more, after all that: still equal
+    a, b = _run_both(lib, fn, first, n_splits=4, min_steps=0)
+    assert torch.equal(a, b)

@@ -22,9 +22,12 @@
 // reduction over the four key groups, and this kernel uses no LDS. Masked keys are read (their page is mapped), but their
 // scores are replaced by -inf and their values by zero before either is used in arithmetic, so what an earlier
 // owner left in a page never reaches a result.
+#include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
+#include "attention_mfma.h"
 
 #ifndef TIS_HD
 #error "compile with -DTIS_HD=<head size>"
@@ -832,12 +835,12 @@ TIS_EXPORT int tis_attention_mfma_tile_columns() { return 16 * TNB; }
 // one, [rows][heads][S][HD] floats and [rows][heads][S] float pairs, S the larger of the two. min_steps > 0: an item
 // uses min(n_splits, its steps of 32 keys / min_steps) splits; a tile uses as many as keep each at most
 // tile_max_steps long; row_splits [rows] receives each row's count.
-TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
-                                  const int* row_seq, const int* positions, const int* items, int n_items, int nb,
-                                  const int* tiles, int n_tiles, void* out, long out_ld, float* part_o,
-                                  float* part_ml, int rows, int n_heads, int n_kv_heads, int head_dim, int page_size,
-                                  int window, float scale, int n_splits, int min_steps, int tile_splits,
-                                  int tile_max_steps, int* row_splits, hipStream_t stream) {
+static int attention_launch(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
+                            const int* row_seq, const int* positions, const int* items, int n_items, int nb,
+                            const int* tiles, int n_tiles, void* out, long out_ld, float* part_o,
+                            float* part_ml, int rows, int n_heads, int n_kv_heads, int head_dim, int page_size,
+                            int window, float scale, int n_splits, int min_steps, int tile_splits,
+                            int tile_max_steps, int* row_splits, hipStream_t stream) {
   if ((n_items == 0 && n_tiles == 0) || rows == 0) return 0;
   if (n_items < 0 || n_tiles < 0 || (n_tiles > 0 && !tiles)) return tis_fail("attention_mfma: bad item counts %d, %d", n_items, n_tiles);
   if (head_dim != HD) return tis_fail("attention_mfma: built for head size %d, called with %d", HD, head_dim);
@@ -915,4 +918,78 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
     rc = tis_launch_status("attention_merge");
   }
   return rc;
+}
+
+TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
+                                  const int* row_seq, const int* positions, const int* items, int n_items, int nb,
+                                  const int* tiles, int n_tiles, void* out, long out_ld, float* part_o,
+                                  float* part_ml, int rows, int n_heads, int n_kv_heads, int head_dim, int page_size,
+                                  int window, float scale, int n_splits, int min_steps, int tile_splits,
+                                  int tile_max_steps, int* row_splits, hipStream_t stream) {
+  return attention_launch(q, q_ld, plane, block_tables, bt_ld, row_seq, positions, items, n_items, nb, tiles, n_tiles,
+                          out, out_ld, part_o, part_ml, rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                          n_splits, min_steps, tile_splits, tile_max_steps, row_splits, stream);
+}
+
+// ---- the same without a workspace argument: partial results in memory that this library owns for good ----
+//
+// The array below is the workspace of tis_attention_mfma_static. Every GPU on which this library's code is loaded holds
+// a copy of it, at an address of its own, until the process ends. In host code the array's name is only a handle for
+// hipGetSymbolAddress: the device address is asked for once per device, with that device current, and kept; kernels,
+// like those of tis_attention_mfma, get the address as an argument.
+static __device__ __align__(256) float scratch[TIS_ATTENTION_STATIC_FLOATS];
+
+static constexpr int kMaxDevices = 64;
+static float* g_scratch_ptr[kMaxDevices];     // null until the device's first call
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return tis_fail("attention_mfma_static: no current device: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return tis_fail("attention_mfma_static: device %d is beyond the %d this library keeps track of", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    float* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return tis_fail("attention_mfma_static: the workspace's address on device %d is not to be had: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+TIS_EXPORT long tis_attention_mfma_static_floats() { return TIS_ATTENTION_STATIC_FLOATS; }
+
+TIS_EXPORT int tis_attention_mfma_static(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
+                                         const int* row_seq, const int* positions, const int* items, int n_items,
+                                         int nb, const int* tiles, int n_tiles, void* out, long out_ld, int rows,
+                                         int n_heads, int n_kv_heads, int head_dim, int page_size, int window,
+                                         float scale, int n_splits, int min_steps, int tile_splits, int tile_max_steps,
+                                         hipStream_t stream) {
+  if ((n_items == 0 && n_tiles == 0) || rows == 0) return 0;
+  if (rows < 0 || n_heads < 1 || n_splits < 1 || tile_splits < 1)
+    return tis_fail("attention_mfma_static: bad sizes rows=%d heads=%d splits=%d, %d", rows, n_heads, n_splits, tile_splits);
+  const int stride = std::max(n_items > 0 ? n_splits : 1, n_tiles > 0 ? tile_splits : 1);
+  float *part_o = nullptr, *part_ml = nullptr;
+  int* row_splits = nullptr;
+  if (stride > 1) {
+    // [rows][heads][stride][HD] partial outputs, [rows][heads][stride] (maximum, sum) pairs, [rows] split counts.
+    // Nothing of it has to start at zero: every slot that the merge reads has been written by this call before.
+    const long o_floats = (long)rows * n_heads * stride * HD, ml_floats = (long)rows * n_heads * stride * 2;
+    const long need = o_floats + ml_floats + rows;
+    if (need > (long)TIS_ATTENTION_STATIC_FLOATS)
+      return tis_fail("attention_mfma_static: %d rows x %d heads x %d splits need %ld floats of partial results; the "
+                      "built-in workspace holds %ld (fewer splits or rows, or tis_attention_mfma with a workspace of "
+                      "the caller's)", rows, n_heads, stride, need, (long)TIS_ATTENTION_STATIC_FLOATS);
+    float* base = nullptr;
+    if (scratch_of_current_device(&base)) return -1;
+    part_o = base;
+    part_ml = base + o_floats;
+    row_splits = reinterpret_cast<int*>(base + o_floats + ml_floats);
+  }
+  return attention_launch(q, q_ld, plane, block_tables, bt_ld, row_seq, positions, items, n_items, nb, tiles, n_tiles,
+                          out, out_ld, part_o, part_ml, rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                          n_splits, min_steps, tile_splits, tile_max_steps, row_splits, stream);
 }

@@ -40,7 +40,7 @@ SOURCES: Dict[str, str] = {
     "gemm_library": "gemm_library.hip",
     "sampling": "sampling.hip",
 }
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "attention_mfma.h"]
 # what a library links beyond the HIP runtime
 LINK: Dict[str, List[str]] = {"gemm_library": ["-lhipblaslt"]}
 

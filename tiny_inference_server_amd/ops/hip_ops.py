@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_float, c_int, c_long, c_void_p
-from typing import Optional
+from typing import NamedTuple, Optional
 
 import numpy as np
 import torch
@@ -185,6 +185,57 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
         nb *= 2
     tiles, steps = cut(tiled, tile_rows)
     return nb, cut(rest, max(1, (16 * nb) // group_size))[0], tiles, steps
+
+
+class AttentionLaunch(NamedTuple):
+    """How one call of the matrix-core attention cuts its keys, and where its partial results lie in the workspace
+    (offsets in floats): [rows][heads][stride][head size] outputs, then [rows][heads][stride] (maximum, sum) pairs,
+    then [rows] split counts."""
+    n_splits: int
+    min_steps: int
+    tile_splits: int
+    tile_max_steps: int
+    stride: int
+    ml_offset: int
+    row_splits_offset: int
+    need_floats: int
+
+
+def attention_launch_plan(n, n_items, n_tiles, tile_steps, single, max_kv_len, n_heads, n_kv_heads, head_dim,
+                          workspace_floats=None) -> AttentionLaunch:
+    """Split counts of one attention call over `n` rows, from the planner's items and tiles; pure host arithmetic."""
+    workspace_floats = _ATTN_WORKSPACE_FLOATS if workspace_floats is None else workspace_floats
+    n_splits, min_steps, tile_splits, tile_max_steps = 1, 0, 1, 1 << 20
+    if n_items:
+        # decoded tokens: every request's keys are cut into the same number of splits, enough to spread a
+        # short batch over the chip. Prompt rows: the grid offers more splits than the chip needs and every
+        # item takes as many as its own length deserves (the kernel decides, from _ATTN_PROMPT_MIN_STEPS),
+        # because the last rows of a long prompt would otherwise run on alone long after the first have finished.
+        target = _ATTN_PROMPT_TARGET_WAVES if (not single and n <= _ATTN_PROMPT_SPLIT_MAX_ROWS) else _ATTN_TARGET_WAVES
+        # a lone request or two: shorter splits still pay, because so few waves would leave most of the chip idle
+        min_keys = _ATTN_MIN_SPLIT_KEYS // 2 if n_items * n_kv_heads <= 8 else _ATTN_MIN_SPLIT_KEYS
+        n_splits = max(1, min(-(-target // (n_items * n_kv_heads)), max_kv_len // min_keys))
+        min_steps = 0 if single else _ATTN_PROMPT_MIN_STEPS
+    if n_tiles:
+        # a tile's keys are cut so that no workgroup walks a chain of steps much longer than an even share of
+        # all tiles' steps: the last rows of a long prompt would otherwise run on alone. Measured at 12 heads
+        # of 128 (tiles / one-wave kernel, us): 2,048 rows from 0: 54 / 69; from 2,048: 99 / 134; from 6,144:
+        # 196 / 260; 4,096 rows: 146 / 202.
+        all_steps, longest = tile_steps
+        share = all_steps * n_kv_heads / _ATTN_TILE_GROUPS
+        tile_max_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
+        most_splits = max(2, _ATTN_TILE_PARTIAL_BYTES // (n * n_heads * head_dim * 4))
+        tile_splits = max(1, min(most_splits, -(-longest // tile_max_steps)))
+        tile_max_steps = max(tile_max_steps, -(-longest // tile_splits))
+    # partial results of split key ranges live in one workspace of fixed size; fewer splits where it
+    # would not suffice
+    most = max(1, (workspace_floats - n) // (n * n_heads * (head_dim + 2)))
+    n_splits, tile_splits = min(n_splits, most), min(tile_splits, most)
+    stride = max(n_splits, tile_splits)
+    ml_offset = n * n_heads * stride * head_dim
+    rs_offset = n * n_heads * stride * (head_dim + 2)
+    return AttentionLaunch(n_splits, min_steps, tile_splits, tile_max_steps, stride, ml_offset, rs_offset,
+                           rs_offset + n if stride > 1 else 0)
 
 
 def _rows_view(t: torch.Tensor, what: str):
@@ -580,39 +631,21 @@ class HipOps:
                     raise KernelError(f"attention: the kernel's tiles hold {built} columns a wave, the planner "
                                       f"assumes {cols}")
             single = items is None and n_tiles == 0
-            n_splits, min_steps, tile_splits, tile_max_steps = 1, 0, 1, 1 << 20
-            if n_items:
-                # decoded tokens: every request's keys are cut into the same number of splits, enough to spread a
-                # short batch over the chip. Prompt rows: the grid offers more splits than the chip needs and every
-                # item takes as many as its own length deserves (the kernel decides, from _ATTN_PROMPT_MIN_STEPS),
-                # because the last rows of a long prompt would otherwise run on alone long after the first have finished.
-                target = _ATTN_PROMPT_TARGET_WAVES if (not single and n <= _ATTN_PROMPT_SPLIT_MAX_ROWS) else _ATTN_TARGET_WAVES
-                # a lone request or two: shorter splits still pay, because so few waves would leave most of the chip idle
-                min_keys = _ATTN_MIN_SPLIT_KEYS // 2 if n_items * n_kv_heads <= 8 else _ATTN_MIN_SPLIT_KEYS
-                n_splits = max(1, min(-(-target // (n_items * n_kv_heads)), batch.max_kv_len // min_keys))
-                min_steps = 0 if single else _ATTN_PROMPT_MIN_STEPS
-            if n_tiles:
-                # a tile's keys are cut so that no workgroup walks a chain of steps much longer than an even share of
-                # all tiles' steps: the last rows of a long prompt would otherwise run on alone. Measured at 12 heads
-                # of 128 (tiles / one-wave kernel, us): 2,048 rows from 0: 54 / 69; from 2,048: 99 / 134; from 6,144:
-                # 196 / 260; 4,096 rows: 146 / 202.
-                all_steps, longest = tile_steps
-                share = all_steps * n_kv_heads / _ATTN_TILE_GROUPS
-                tile_max_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
-                most_splits = max(2, _ATTN_TILE_PARTIAL_BYTES // (n * n_heads * head_dim * 4))
-                tile_splits = max(1, min(most_splits, -(-longest // tile_max_steps)))
-                tile_max_steps = max(tile_max_steps, -(-longest // tile_splits))
-            # partial results of split key ranges live in one workspace of fixed size; fewer splits where it
-            # would not suffice
-            most = max(1, (_ATTN_WORKSPACE_FLOATS - n) // (n * n_heads * (head_dim + 2)))
-            n_splits, tile_splits = min(n_splits, most), min(tile_splits, most)
-            stride = max(n_splits, tile_splits)
+            lp = attention_launch_plan(n, n_items, n_tiles, tile_steps, single, batch.max_kv_len, n_heads, n_kv_heads,
+                                       head_dim)
+            n_splits, min_steps, tile_splits, tile_max_steps = lp.n_splits, lp.min_steps, lp.tile_splits, lp.tile_max_steps
             part_o = part_ml = row_splits = None
-            if stride > 1:
+            if lp.stride > 1:
+                if lp.need_floats > self._workspace.numel():
+                    raise KernelError(f"attention: {lp.need_floats} floats of partial results for a workspace of "
+                                      f"{self._workspace.numel()}")
                 part_o = self._workspace
-                part_ml = self._workspace[n * n_heads * stride * head_dim:]
+                part_ml = self._workspace[lp.ml_offset:]
                 if not single:
-                    row_splits = self._workspace[n * n_heads * stride * (head_dim + 2):]
+                    row_splits = self._workspace[lp.row_splits_offset:]
+            if lines.numel() < 2 * (n_items + n_tiles) or lines.dtype != torch.int32 or not lines.is_contiguous():
+                raise KernelError(f"attention: the work list holds {lines.numel()} entries for {n_items} items and "
+                                  f"{n_tiles} tiles")
             lib.tis_attention_mfma(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0),
                                    _ptr(batch.row_seq), _ptr(batch.positions), _ptr(items), n_items, nb, _ptr(tiles),
                                    n_tiles, _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), n, n_heads,

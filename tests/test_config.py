@@ -96,9 +96,9 @@ def test_spec_is_built_from_the_config_alone():
     sa, sb = build(a), build(b)
     assert len(sa.layers) == 3 and len(sb.layers) == 5 and [s.lag for s in sb.stages] == [0, 1, 2]
     assert sa.lm_head == sa.embedding and sb.lm_head == "lm_head.weight"
-    ma, mb = sa.layers[0].mixer.params, sb.layers[0].mixer.params
+    ma, mb = sa.layers[0].part("mixer").params, sb.layers[0].part("mixer").params
     assert (ma["n_heads"], ma["n_kv_heads"], ma["head_dim"]) == (8, 2, 8)
     assert (mb["n_heads"], mb["n_kv_heads"], mb["head_dim"]) == (3, 1, 32)
     assert ma["position"].params["base"] == 1e4 and mb["position"].params["base"] == 5e5
-    assert sa.layers[0].mixer_norm.params["eps"] == 2e-8 and sb.layers[0].mixer_norm.params["eps"] == 1e-5
-    assert sb.layers[4].mixer.tensors["q"] == "mtp_heads_list.1.trans_block.att.q_proj.weight"
+    assert sa.layers[0].part("mixer_norm").params["eps"] == 2e-8 and sb.layers[0].part("mixer_norm").params["eps"] == 1e-5
+    assert sb.layers[4].part("mixer").tensors["q"] == "mtp_heads_list.1.trans_block.att.q_proj.weight"

@@ -86,7 +86,8 @@ def test_attention_mixer_and_block(name, dtype, tol, n_heads, n_kv, hd):
     norm = lambda n: PartSpec("norm", "rmsnorm_l2", {"width": D, "eps": eps}, {"gain": n})
     ffn = PartSpec("feed_forward", "swiglu", {"d_model": D, "hidden": Fh},
                    {"gate": "b.ffn.swig.linear1.weight", "up": "b.ffn.swig.linear2.weight", "down": "b.ffn.fc.weight"})
-    layer = LayerSpec("prenorm_residual", mixer, norm("b.att.rms_norm_att.scale"), ffn, norm("b.rms_norm_ffn.scale"))
+    layer = LayerSpec("prenorm_residual", {"mixer": mixer, "mixer_norm": norm("b.att.rms_norm_att.scale"),
+                                           "feed_forward": ffn, "feed_forward_norm": norm("b.rms_norm_ffn.scale")})
     t = {"b.att.q_proj.weight": rnd((D, D), 10, D ** -0.5), "b.att.kv_proj.weight": rnd((D, 2 * n_kv * hd), 11, D ** -0.5),
          "b.att.linear_proj.weight": rnd((D, D), 12, D ** -0.5), "b.ffn.swig.linear1.weight": rnd((D, Fh), 13, D ** -0.5),
          "b.ffn.swig.linear2.weight": rnd((D, Fh), 14, D ** -0.5), "b.ffn.fc.weight": rnd((Fh, D), 15, Fh ** -0.5),
@@ -167,7 +168,8 @@ def toy_spec(cfg):
         mixer = PartSpec("mixer", "toy_decay", {"d_model": cfg.d_model, "decay": cfg.decay}, {"w": f"l{l}.mix.w"})
         ffn = PartSpec("feed_forward", "swiglu", {"d_model": cfg.d_model, "hidden": cfg.hidden},
                        {"gate": f"l{l}.g", "up": f"l{l}.u", "down": f"l{l}.d"})
-        layers.append(LayerSpec("prenorm_residual", mixer, norm(f"l{l}.n1"), ffn, norm(f"l{l}.n2")))
+        layers.append(LayerSpec("prenorm_residual", {"mixer": mixer, "mixer_norm": norm(f"l{l}.n1"),
+                                                     "feed_forward": ffn, "feed_forward_norm": norm(f"l{l}.n2")}))
     # the run order is data: layer 0, layer 1, then layer 0 again with a state of its own
     stage = StageSpec("trunk", 0, PartSpec("stage_input", "token_embedding"),
                       (LayerCall(0), LayerCall(1), LayerCall(0)), norm("out"))
@@ -190,6 +192,7 @@ def toy_plain(ids, w, cfg):
 
 def test_toy_mixer_with_state_is_registered_built_and_stepped():
     ARCHITECTURES.register("ToyStateModel", Architecture("ToyStateModel", ToyConfig, toy_spec), replace=True)
+    MIXERS.register("toy_decay", ToyDecayMixer, replace=True)
     cfg = ToyConfig(d_model=48, vocab_size=101, hidden=80, decay=0.7)
     w = random_tensors(cfg, 9, std=0.1, gain_jitter=0.1, dtype="float32")
     eng = Engine(config=cfg, tensors=w, dtype="float32", page_size=16, max_tokens=64, max_requests=3)
@@ -206,6 +209,110 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
     MIXERS.unregister("toy_decay")
 
 
+# ---- toy arrangements: a block with no feed-forward, and a block with two mixers, each with a cache of its own ------
+
+def register_toy_arrangements():
+    from tiny_inference_server_amd.parts import Arrangement
+
+    @ARRANGEMENTS.register("toy_mixer_only", replace=True)
+    class ToyMixerOnly(Arrangement):
+        """x = x + mixer(norm(x)): no feed-forward at all."""
+        part_names = ("norm", "mixer")
+
+        def forward(self, x, ctx):
+            return self.parts["mixer"].forward(self.parts["norm"](x), ctx.of("mixer"), residual=x)
+
+    @ARRANGEMENTS.register("toy_two_mixers", replace=True)
+    class ToyTwoMixers(Arrangement):
+        """x = x + attention(norm(x)) + decay(norm(x)): two mixers read the same normed rows; one has pages, the other
+        a state slot."""
+        part_names = ("norm", "attention", "decay")
+
+        def forward(self, x, ctx):
+            a = self.parts["norm"](x)
+            x = self.parts["attention"].forward(a, ctx.of("attention"), residual=x)
+            return self.parts["decay"].forward(a, ctx.of("decay"), residual=x)
+
+
+def toy_arrangement_spec(cfg):
+    from tiny_inference_server_amd.architectures.gqa_mtp import _block, _norm
+    layers = []
+    for l in range(3):
+        blk = _block(cfg, f"transformer_block_list.{l}.")
+        norm, att = blk.part("mixer_norm"), blk.part("mixer")
+        decay = PartSpec("mixer", "toy_decay", {"d_model": cfg.d_model, "decay": 0.6}, {"w": f"l{l}.decay.w"})
+        if l == 0:
+            layers.append(LayerSpec("toy_mixer_only", {"norm": norm, "mixer": att}))
+        elif l == 1:
+            layers.append(LayerSpec("toy_two_mixers", {"norm": norm, "attention": att, "decay": decay}))
+        else:
+            layers.append(blk)
+    stage = StageSpec("trunk", 0, PartSpec("stage_input", "token_embedding"), tuple(LayerCall(l) for l in range(3)),
+                      _norm(cfg, "rms_out.scale"))
+    return ModelSpec(cfg.d_model, cfg.vocab_size, cfg.max_context, tuple(layers), (stage,), "embedding.weight", "embedding.weight")
+
+
+def toy_arrangement_plain(ids, w, cfg):
+    T, D, NH, G = len(ids), cfg.d_model, cfg.n_heads, cfg.group_size
+    hd, pos = D // NH, torch.arange(len(ids))
+    x = w["embedding.weight"][torch.tensor(ids)]
+
+    def attention(a, pre):
+        q = pm.apply_rope((a @ w[pre + "att.q_proj.weight"]).view(T, NH, hd), pos, cfg.rope_base)
+        k, v = (a @ w[pre + "att.kv_proj.weight"]).view(T, 2, NH // G, hd).unbind(1)
+        return pm.causal_gqa_attention(q, pm.apply_rope(k, pos, cfg.rope_base), v, G).reshape(T, D) @ w[pre + "att.linear_proj.weight"]
+
+    for l in range(3):
+        pre = f"transformer_block_list.{l}."
+        a = pm.rms_norm(x, w[pre + "att.rms_norm_att.scale"], cfg.rms_eps)
+        x = x + attention(a, pre)
+        if l == 1:
+            s, rows = torch.zeros(D, dtype=torch.float64), []
+            for r in range(T):
+                s = 0.6 * s + a[r]
+                rows.append(s)
+            x = x + torch.stack(rows) @ w["l1.decay.w"]
+        if l == 2:
+            f = pm.rms_norm(x, w[pre + "rms_norm_ffn.scale"], cfg.rms_eps)
+            x = x + pm.swiglu_ffn(f, w[pre + "ffn.swig.linear1.weight"], w[pre + "ffn.swig.linear2.weight"], w[pre + "ffn.fc.weight"])
+    return pm.rms_norm(x, w["rms_out.scale"], cfg.rms_eps) @ w["embedding.weight"].T
+
+
+def test_toy_blocks_without_feed_forward_and_with_two_mixers():
+    """Which parts a block has is the arrangement's business. From here, with no dummy parts and no change to the
+    framework: a block of norm and attention alone, and a block whose two mixers (attention with pages, a recurrence
+    with a state slot) each get a cache of their own; beside the built-in block. The loader asks for exactly the
+    tensors these parts name."""
+    from tiny_inference_server_amd.config import GqaMtpConfig
+    from tiny_inference_server_amd.weights.loader import spec_tensors
+    register_toy_arrangements()
+    MIXERS.register("toy_decay", ToyDecayMixer, replace=True)
+    cfg = GqaMtpConfig(d_model=80, vocab_size=131, max_context=256, rope_base=1e4, n_heads=5, n_layers=3, ffn_hidden=56,
+                       group_size=5, mtp_heads=0, architecture="ToyArrangements")
+    ARCHITECTURES.register("ToyArrangements", Architecture("ToyArrangements", GqaMtpConfig, toy_arrangement_spec), replace=True)
+    names = set(spec_tensors(toy_arrangement_spec(cfg)))
+    assert "l1.decay.w" in names and not any(n.startswith(("transformer_block_list.0.ffn", "transformer_block_list.1.ffn",
+                                                            "transformer_block_list.0.rms_norm_ffn")) for n in names)
+    w = {n: 0.1 * rnd(sh, 40 + i) if len(sh) > 1 else 1 + 0.1 * rnd(sh, 40 + i)
+         for i, (n, sh) in enumerate(sorted(spec_tensors(toy_arrangement_spec(cfg)).items()))}
+    eng = Engine(config=cfg, tensors=w, dtype="float32", page_size=16, max_tokens=256, max_requests=3)
+    needs = eng.model.cache_needs()
+    assert sorted(needs) == ["trunk.0", "trunk.1:attention", "trunk.1:decay", "trunk.2"]
+    assert isinstance(needs["trunk.1:decay"], StateNeed) and len(eng.cache.groups) == 1
+    w64 = {k: v.double() for k, v in w.items()}
+    reqs = {"a": H.random_ids(131, 41, 5), "b": H.random_ids(131, 19, 6)}
+    for trace in (H.whole_trace(reqs), H.mixed_trace(reqs, 2, 7)[0], H.portions_trace({"a": reqs["a"]}, 3)):
+        got, _ = H.run_trace(eng, trace, heads=False)
+        assert got
+        for (rid, p), lg in got.items():
+            want = toy_arrangement_plain(reqs[rid], w64, cfg)[p]
+            assert (lg.double() - want).abs().max() <= 2e-5 * max(1.0, want.abs().max()), (rid, p)
+    ARCHITECTURES.unregister("ToyArrangements")
+    MIXERS.unregister("toy_decay")
+    ARRANGEMENTS.unregister("toy_mixer_only")
+    ARRANGEMENTS.unregister("toy_two_mixers")
+
+
 # ---- layers with different cache needs in one model: a sliding window beside full attention ----------------------
 
 def windowed_spec(cfg, windows):
@@ -214,8 +321,8 @@ def windowed_spec(cfg, windows):
     layers = []
     for l, win in enumerate(windows):
         blk = _block(cfg, f"transformer_block_list.{l}.")
-        mixer = dataclasses.replace(blk.mixer, params={**blk.mixer.params, "window": win})
-        layers.append(dataclasses.replace(blk, mixer=mixer))
+        mixer = blk.part("mixer")
+        layers.append(blk.with_part("mixer", dataclasses.replace(mixer, params={**mixer.params, "window": win})))
     stage = StageSpec("trunk", 0, PartSpec("stage_input", "token_embedding"), tuple(LayerCall(l) for l in range(len(windows))),
                       _norm(cfg, "rms_out.scale"))
     return ModelSpec(cfg.d_model, cfg.vocab_size, cfg.max_context, tuple(layers), (stage,), "embedding.weight", "embedding.weight")
@@ -327,14 +434,15 @@ def routed_spec(cfg, n_experts, stretch):
         blk = _block(cfg, f"transformer_block_list.{l}.")
         pos = PartSpec("position", "toy_stretched_rotary", {"head_dim": cfg.head_dim, "base": cfg.rope_base,
                                                             "max_context": cfg.max_context, "stretch": stretch})
-        mixer = dataclasses.replace(blk.mixer, params={**blk.mixer.params, "position": pos})
+        mixer = dataclasses.replace(blk.part("mixer"), params={**blk.part("mixer").params, "position": pos})
         names = {"router": f"l{l}.router"}
         for e in range(n_experts):
             names.update({f"gate{e}": f"l{l}.e{e}.g", f"up{e}": f"l{l}.e{e}.u", f"down{e}": f"l{l}.e{e}.d"})
         ffn = PartSpec("feed_forward", "toy_top1_experts",
                        {"d_model": cfg.d_model, "hidden": cfg.ffn_hidden, "n_experts": n_experts}, names)
         # the second layer keeps the built-in dense feed-forward: parts are chosen layer by layer
-        layers.append(dataclasses.replace(blk, mixer=mixer, feed_forward=ffn if l != 1 else blk.feed_forward))
+        blk = blk.with_part("mixer", mixer)
+        layers.append(blk.with_part("feed_forward", ffn) if l != 1 else blk)
     stage = StageSpec("trunk", 0, PartSpec("stage_input", "token_embedding"), tuple(LayerCall(l) for l in range(cfg.n_layers)),
                       _norm(cfg, "rms_out.scale"))
     return ModelSpec(cfg.d_model, cfg.vocab_size, cfg.max_context, tuple(layers), (stage,), "embedding.weight", "embedding.weight")

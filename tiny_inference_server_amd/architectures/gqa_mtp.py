@@ -30,8 +30,9 @@ def _block(cfg, prefix):
     ffn = PartSpec("feed_forward", "swiglu", {"d_model": cfg.d_model, "hidden": cfg.ffn_hidden},
                    {"gate": prefix + "ffn.swig.linear1.weight", "up": prefix + "ffn.swig.linear2.weight",
                     "down": prefix + "ffn.fc.weight"})
-    return LayerSpec("prenorm_residual", mixer, _norm(cfg, prefix + "att.rms_norm_att.scale"), ffn,
-                     _norm(cfg, prefix + "rms_norm_ffn.scale"))
+    return LayerSpec("prenorm_residual", {"mixer_norm": _norm(cfg, prefix + "att.rms_norm_att.scale"), "mixer": mixer,
+                                          "feed_forward_norm": _norm(cfg, prefix + "rms_norm_ffn.scale"),
+                                          "feed_forward": ffn})
 
 
 def build_spec(cfg: GqaMtpConfig) -> ModelSpec:

@@ -193,7 +193,7 @@ class Engine:
                 step = materialize(plan, self.device)
             else:
                 step = build_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
-                                        self.device, self.spec.max_context, getattr(self.ops, "plan_rows", None))
+                                        self.device, self.spec.max_context, self.model.plan_rows)
             outs = self.model.forward(step, self.cache)
         n = sum(len(e.want) for e in batch_entries)
         head_logits = head_valid = None
@@ -254,7 +254,7 @@ class Engine:
         pages = max((max(len(g.tables[e.slot]) for e in batch_entries) for g in self.cache.groups.values()), default=1)
         width = -(-pages // self.graph_table_pages) * self.graph_table_pages
         plan = plan_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
-                               self.spec.max_context, getattr(self.ops, "plan_rows", None), table_width=width)
+                               self.spec.max_context, self.model.plan_rows, table_width=width)
         # what the host decides from, beyond the arrays' shapes
         key = ("step", width, plan.layout(),
                tuple((pl["max_rows"], pl["keep_count"], pl["previous_rows"], tuple(pl["valid"])) for pl in plan.plans))
@@ -292,7 +292,7 @@ class Engine:
             self.graph_replays += 1
             return graph.run_same_requests(batch_entries)
         plan = plan_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
-                               self.spec.max_context, getattr(self.ops, "plan_rows", None), table_width=width)
+                               self.spec.max_context, self.model.plan_rows, table_width=width)
         if graph is None:
             seen = self._graph_seen.get(key, 0)
             self._graph_seen[key] = seen + 1

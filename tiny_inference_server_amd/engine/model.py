@@ -33,28 +33,41 @@ class Model:
         # step's device arrays alone, never on host values that change from step to step
         parts = list(self.inputs) + list(self.out_norms)
         for blk in self.layers:
-            parts += [getattr(blk, n) for n in ("mixer", "mixer_norm", "ffn", "ffn_norm") if hasattr(blk, n)] or [blk]
+            # an arrangement that builds no parts of its own answers for itself
+            parts += list(getattr(blk, "parts", {}).values()) or [blk]
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
+        # host planning that parts ask for, once per distinct key (layers of one shape share a plan)
+        self._planners = {}
+        for p in parts:
+            key = p.plan_key() if hasattr(p, "plan_key") else None
+            if key is not None:
+                self._planners.setdefault(key, p)
         self.lags = [st.lag for st in spec.stages]
         self.max_lag = max(self.lags)
         self.reads_previous = [bool(getattr(part_class(st.input), "reads_previous", False)) for st in spec.stages]
         if self.reads_previous and self.reads_previous[0]:
             raise ValueError("the first stage cannot read a previous stage")
-        # cache keys: one per call unless the call names another's
-        self.call_keys: List[List[str]] = []
+        # cache keys: one per call and mixer part unless the call names another's; a block with one mixer uses the
+        # call's key as it is, a block with several appends the part's name
+        self.call_keys: List[List[Dict[str, str]]] = []
         self.needs: Dict[str, object] = {}
         for st in spec.stages:
             keys = []
             for i, call in enumerate(st.calls):
-                key = call.cache or f"{st.name}.{i}"
-                need = part_class(spec.layers[call.layer].mixer).cache_need(spec.layers[call.layer].mixer.params)
-                if call.writes_cache or key not in self.needs:
-                    if key in self.needs and self.needs[key] != need:
-                        raise ValueError(f"cache {key!r} is shared by layers that need different things: "
-                                         f"{self.needs[key]} and {need}")
-                    if need is not None:
-                        self.needs[key] = need
-                keys.append(key)
+                base = call.cache or f"{st.name}.{i}"
+                mixers = spec.layers[call.layer].mixers()
+                per_part = {}
+                for name, mixer in mixers:
+                    key = base if len(mixers) == 1 else f"{base}:{name}"
+                    need = part_class(mixer).cache_need(mixer.params)
+                    if call.writes_cache or key not in self.needs:
+                        if key in self.needs and self.needs[key] != need:
+                            raise ValueError(f"cache {key!r} is shared by layers that need different things: "
+                                             f"{self.needs[key]} and {need}")
+                        if need is not None:
+                            self.needs[key] = need
+                    per_part[name] = key
+                keys.append(per_part)
             self.call_keys.append(keys)
         self.state_keys: List[Optional[str]] = []
         for st in spec.stages:
@@ -67,21 +80,36 @@ class Model:
     def cache_needs(self) -> Dict[str, object]:
         return dict(self.needs)
 
+    def plan_rows(self, seq_rows, add):
+        """Host planning of every part that asks for it, for one stage's rows: {name: (packed array id, values...)}."""
+        plans = {}
+        for part in self._planners.values():
+            plans.update(part.plan_rows(seq_rows, add))
+        return plans
+
+    def _bind(self, ctx, key, cache):
+        need = self.needs.get(key)
+        if isinstance(need, PagedKvNeed):
+            ctx.group = cache.group_of[key]
+            ctx.plane = cache.groups[ctx.group].plane(key)
+        elif isinstance(need, StateNeed):
+            ctx.state = cache.states[key]
+        return ctx
+
     def _run_stage(self, j, step, cache, prev):
         st, b = self.spec.stages[j], step.stages[j]
         state = cache.states.get(self.state_keys[j]) if self.state_keys[j] else None
         x = self.inputs[j].forward(b, prev, self.shared, state)
         if b.n_rows:
             for i, call in enumerate(st.calls):
-                key = self.call_keys[j][i]
-                need = self.needs.get(key)
+                keys = self.call_keys[j][i]
                 # the rows going into a layer are replaced by its result: the layer may overwrite them
                 ctx = CallContext(batch=b, writes_cache=call.writes_cache, residual_is_spent=True)
-                if isinstance(need, PagedKvNeed):
-                    ctx.group = cache.group_of[key]
-                    ctx.plane = cache.groups[ctx.group].plane(key)
-                elif isinstance(need, StateNeed):
-                    ctx.state = cache.states[key]
+                if len(keys) == 1:
+                    self._bind(ctx, next(iter(keys.values())), cache)
+                elif keys:
+                    ctx.bindings = {name: self._bind(CallContext(batch=b, writes_cache=call.writes_cache), key, cache)
+                                    for name, key in keys.items()}
                 x = self.layers[call.layer].forward(x, ctx)
             x = self.out_norms[j](x)
         return x

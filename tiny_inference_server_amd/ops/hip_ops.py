@@ -273,27 +273,23 @@ class HipOps:
             self.gemm_library = library("gemm_library")
             with torch.cuda.device(self.device):
                 self.gemm_library.tis_gemm_library_init()
-        self._attn_groups = set()          # group sizes of the attention mixers built on these ops
         self._attn_mfma = {}               # head size -> library
         # partial results of split key ranges: one buffer of fixed size that never moves (captured graphs hold its address)
         self._workspace = torch.empty(_ATTN_WORKSPACE_FLOATS, dtype=torch.float32, device=self.device) \
             if dtype == torch.bfloat16 else None
 
     # ---- planning on the host --------------------------------------------------------------------------
-    def register_attention(self, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
-        """An attention mixer announces its shape, so that each step's work items are planned once, up front."""
-        self._attn_groups.add((n_heads // n_kv_heads, tile_columns(head_dim), n_kv_heads))
-
-    def plan_rows(self, seq_rows, add):
-        """Called while a step's arrays are packed: returns {name: (packed array id, host values...)}."""
+    def plan_attention(self, n_heads: int, n_kv_heads: int, head_dim: int, seq_rows, add):
+        """An attention mixer's host planning, called while a step's arrays are packed: the work items of the
+        matrix-core kernels for the step's rows. Returns {name: (packed array id, host values...)}."""
         plans = {}
         if self.dtype == torch.bfloat16:
-            for group, cols, kvh in sorted(self._attn_groups):
-                nb, items, tiles, steps = attention_items(seq_rows, group, cols, kvh)
-                if nb <= 4 and (len(items) or len(tiles)):
-                    # one array: the items' lines, then the tiles'
-                    plans[("attention_items", group, cols, kvh)] = (add(np.concatenate((items, tiles))), len(items),
-                                                                    nb, len(tiles), steps)
+            group, cols = n_heads // n_kv_heads, tile_columns(head_dim)
+            nb, items, tiles, steps = attention_items(seq_rows, group, cols, n_kv_heads)
+            if nb <= 4 and (len(items) or len(tiles)):
+                # one array: the items' lines, then the tiles'
+                plans[("attention_items", group, cols, n_kv_heads)] = (add(np.concatenate((items, tiles))), len(items),
+                                                                       nb, len(tiles), steps)
         return plans
 
     # ---- helpers -------------------------------------------------------------------------------------

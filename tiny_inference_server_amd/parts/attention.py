@@ -56,10 +56,17 @@ class GqaAttention:
         self.w_qkv = to_compute(ops, w)
         self.w_o = to_compute(ops, tensors.of(spec, "o").t())
         self.q_width = self.n_heads * self.head_dim
-        if hasattr(ops, "register_attention"):
-            ops.register_attention(self.n_heads, self.n_kv_heads, self.head_dim)
 
     fuses_norm = True
+
+    # work lists for the attention kernels are made on the host, once per step and attention shape
+    def plan_key(self):
+        if not hasattr(self.ops, "plan_attention"):
+            return None
+        return ("attention", self.n_heads, self.n_kv_heads, self.head_dim)
+
+    def plan_rows(self, seq_rows, add):
+        return self.ops.plan_attention(self.n_heads, self.n_kv_heads, self.head_dim, seq_rows, add)
 
     def forward(self, x, ctx, residual=None, norm=None):
         ops, b = self.ops, ctx.batch

@@ -22,14 +22,18 @@ feed-forward    forward(x, residual=None) -> y
                 a mixer or feed-forward with the class attribute fuses_norm = True takes forward(..., norm=part)
                 instead: x arrives un-normed and the part applies `norm` itself, fused into its first product
                 where it can
-arrangement     __init__(layer_spec, parts...), forward(x, ctx) -> x      how norm, mixer and feed-forward are wired
+arrangement     part_names (the names of the parts it wires), __init__(layer_spec, tensors, ops) (the base class
+                builds self.parts), forward(x, ctx) -> x; a mixer part gets ctx.of(its name)
+planning        a part may offer plan_key() -> hashable | None and plan_rows(seq_rows, add) -> {name: (array id,
+                host values...)}: host-side work lists for its kernels, made once per step and distinct key while the
+                step's arrays are packed, found again in batch.extras[name]
 stage input     state_need(params) -> StateNeed | None classmethod
                 forward(batch, previous_output, previous_batch, shared, state) -> rows
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Optional
+from typing import Any, Dict, Optional, Tuple
 
 from ..config.registry import Registry
 
@@ -43,13 +47,37 @@ STAGE_INPUTS: Registry = Registry("stage input")
 
 @dataclass
 class CallContext:
-    """What one layer call sees of the step: the rows' metadata and the cache that belongs to the call."""
+    """What one layer call sees of the step: the rows' metadata and the cache that belongs to the call.
+
+    A block with one mixer finds that mixer's cache right here. A block with several asks `ctx.of(part name)` for
+    each mixer's own context (same batch, that part's cache)."""
     batch: Any                       # engine.batch.StageBatch
     group: Optional[str] = None      # page group of the call's cache, for paged needs
     plane: Any = None                # [pages, 2, kv heads, page size, head size] for paged needs
     state: Any = None                # [max requests, *shape] for state needs
     writes_cache: bool = True
     residual_is_spent: bool = False  # the caller will not read the residual it passes again: it may be overwritten
+    bindings: Optional[Dict[str, "CallContext"]] = None     # per mixer part of the block
+
+    def of(self, part_name: str) -> "CallContext":
+        if self.bindings and part_name in self.bindings:
+            return self.bindings[part_name]
+        return self
+
+
+class Arrangement:
+    """Base of block arrangements: builds the parts the spec names and checks them against what the class declares.
+
+    part_names: the names this arrangement wires together (None: whatever the spec brings). After construction
+    `self.parts[name]` is the built part."""
+    part_names: Optional[Tuple[str, ...]] = None
+
+    def __init__(self, layer_spec, tensors, ops):
+        if self.part_names is not None and set(layer_spec.parts) != set(self.part_names):
+            raise ValueError(f"a {layer_spec.arrangement!r} block is made of {sorted(self.part_names)}, "
+                             f"its spec brings {sorted(layer_spec.parts)}")
+        self.ops = ops
+        self.parts = {name: build_part(spec, tensors, ops) for name, spec in layer_spec.parts.items()}
 
 
 class Tensors:

@@ -5,7 +5,7 @@ and runs the spec and never asks which architecture it came from.
 
 * `PartSpec`      one part: its role and kind (a registry and a name in it), its sizes and
                   constants, and the full names of the tensors it owns.
-* `LayerSpec`     one block: an arrangement kind and the parts it arranges.
+* `LayerSpec`     one block: an arrangement kind and the parts it arranges, by the names the arrangement gives them.
 * `LayerCall`     one entry of the run order: which layer runs and whose cache it uses.
 * `StageSpec`     one pass over the rows of a step: where its input comes from,
                   the ordered calls, the closing norm.  A stage with `lag` j runs
@@ -29,11 +29,23 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    arrangement: str              # block arrangement kind, e.g. "prenorm_residual"
-    mixer: PartSpec
-    mixer_norm: PartSpec
-    feed_forward: PartSpec
-    feed_forward_norm: PartSpec
+    """One block. Which parts a block has is the arrangement's business: it declares their names, and the loader,
+    the cache manager and the graph check walk whatever is there. A block may have no feed-forward, two mixers,
+    norms in other places; every part whose role is "mixer" gets a cache of its own if its kind asks for one."""
+    arrangement: str                      # block arrangement kind, e.g. "prenorm_residual"
+    parts: Mapping[str, PartSpec]         # the arrangement's name for the part -> the part
+
+    def part(self, name: str) -> PartSpec:
+        try:
+            return self.parts[name]
+        except KeyError:
+            raise KeyError(f"a {self.arrangement!r} block has no part {name!r}; it has {sorted(self.parts)}") from None
+
+    def with_part(self, name: str, spec: PartSpec) -> "LayerSpec":
+        return LayerSpec(self.arrangement, {**self.parts, name: spec})
+
+    def mixers(self) -> Tuple[Tuple[str, PartSpec], ...]:
+        return tuple((n, p) for n, p in self.parts.items() if p.role == "mixer")
 
 
 @dataclass(frozen=True)

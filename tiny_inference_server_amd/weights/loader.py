@@ -35,7 +35,7 @@ def spec_tensors(spec) -> Dict[str, Tuple[int, ...]]:
     add(spec.embedding, (spec.vocab_size, spec.d_model))
     add(spec.lm_head, (spec.vocab_size, spec.d_model))
     for layer in spec.layers:
-        for part in (layer.mixer, layer.mixer_norm, layer.feed_forward, layer.feed_forward_norm):
+        for part in layer.parts.values():
             for n, s in part_tensors(part).items():
                 add(n, s)
     for stage in spec.stages:

@@ -80,6 +80,10 @@ def main() -> int:
     from tiny_inference_server_amd.engine import Engine
     from tiny_inference_server_amd.weights import random_tensors
 
+    def say(what):
+        # progress on stderr, flushed: names the phase a run was in if it ends without its line
+        print(f"[bench] {what}", file=sys.stderr, flush=True)
+
     cfg_full = size_config(a.size)
     cfg = cfg_full
     if a.layers and a.layers != cfg_full.n_layers:
@@ -141,19 +145,23 @@ def main() -> int:
                 best = dt if best is None else min(best, dt)
         return best
 
+    say(f"{a.size}, {cfg.n_layers} layers, {a.dtype}: decode at batch {a.batch}, context {a.context}")
     value, sec_per_step = decode_rate(a.batch, a.steps, a.warmup)
     elem = 2 if a.dtype == "bfloat16" else 4
     with_table, _ = matmul_params(cfg, heads)
     step_bytes = with_table * elem + a.batch * (a.context - a.steps // 2) * kv_bytes_per_token(cfg, heads, elem)
     achieved = step_bytes / sec_per_step / 1e9
+    say(f"prefill of {a.prefill_tokens} tokens")
     pt = prefill_rate(a.prefill_tokens)
     dkey = "bf16" if a.dtype == "bfloat16" else "fp32"
     pf = prefill_flops(cfg, a.prefill_tokens, heads)
     pts = {}
     for B in points:
+        say(f"decode at batch {B}")
         pts[f"decode_b{B}"] = round(decode_rate(B, max(8, a.steps // 2), max(2, a.warmup // 2))[0], 1)
     if trunk is not None:
         # the reference's "plain" decode runs no prediction heads; the same here, for comparison with its numbers
+        say(f"decode at batch {a.batch} without the prediction heads")
         pts[f"decode_b{a.batch}_trunk_only"] = round(decode_rate(a.batch, a.steps, a.warmup, trunk)[0], 1)
     line = {
         "metric": f"decode tok/s at batch {a.batch} ({a.size}, {dkey}); prefill tok/s at {a.prefill_tokens:,} tokens",

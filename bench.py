@@ -6,7 +6,19 @@
 A step is one decode step: every live request advances by one token through the whole model (trunk, the
 prediction heads unless --trunk-only, output table, sampling, read-back of the tokens). One JSON line is
 printed: decoded tokens a second at the given batch, the prefill of 2,048 tokens, the decode step's
-bandwidth against the HBM peak, and decode at batch 1 and 64.
+bandwidth against the HBM peak, decode at batch 1 and 64, and the same batch-8 decode driven by the scheduler
+with the reference's sampling options instead of by the step function with arg-max.
+
+Two more workloads run whole requests through the scheduler (admission, portions under the token budget, sampling
+with temperature, top-k, top-p and repetition penalty, finishing, pages given back):
+
+    python bench.py --workload serve --size 2.1B     64 requests at once, prompts of 128..4096 tokens, 256 new each
+    python bench.py --workload mixed --size 7B       64 requests decoding at contexts of 512..8192 while 2,048-token
+                                                     portions of further prompts run in the same steps
+
+Each prints one line of the same form; `value` is generated tokens a second over the whole run (serve) or over the
+steps that hold 64 decoding requests and a portion (mixed), `roofline` the sum of the steps' floors (the larger of
+bytes / HBM peak and flops / matrix peak) over the sum of their times.
 """
 from __future__ import annotations
 
@@ -51,6 +63,180 @@ def prefill_flops(cfg, T: int, heads: bool):
     return linear + attention
 
 
+# the reference's sampling options for its runs (server.py:515-516, evals.py:120)
+SAMPLING = dict(temperature=0.9, top_k=50, top_p=0.95, rep_penalty=1.1)
+
+
+def step_floor(cfg, heads, elem, n_tokens, kv_tokens, attn_pairs, dkey):
+    """Seconds one step needs at the least: its bytes at the HBM peak or its flops at the matrix peak."""
+    with_table, without = matmul_params(cfg, heads)
+    planes = cfg.n_layers + (cfg.mtp_heads if heads else 0)
+    byts = with_table * elem + kv_tokens * kv_bytes_per_token(cfg, heads, elem)
+    flops = 2.0 * without * n_tokens + planes * 4.0 * cfg.n_heads * cfg.head_dim * attn_pairs
+    return max(byts / (HBM_GBS * 1e9), flops / PEAK_FLOPS[dkey]), byts, flops
+
+
+def scheduler_decode_rate(engine, a, cfg, gen):
+    """Tokens a second of `a.steps` decode steps at batch `a.batch` near the context length, through the scheduler."""
+    import torch
+
+    from tiny_inference_server_amd.engine.scheduler import Request, Scheduler
+    from tiny_inference_server_amd.sampling.params import SamplingParams
+    sched = Scheduler(engine, max_batch=a.batch, token_budget=2048 + a.batch, plan="final")
+    # a request that has its prompt in decodes while the others' portions are still fed: room for those tokens too
+    early = a.batch * -(-a.context // 2048) + 2
+    start_len = max(1, a.context - a.steps - a.warmup - early)
+    for i in range(a.batch):
+        ids = torch.randint(0, cfg.vocab_size, (start_len,), generator=gen).tolist()
+        sched.submit(Request(ids, SamplingParams(max_new_tokens=a.steps + a.warmup + early, seed=a.seed + i,
+                                                 ignore_eos=True, **SAMPLING)))
+    sched.admit()
+    while any(r.fed < r.prompt_len for r in sched.active):      # prompts, in portions; the last portion samples
+        sched.step()
+    for _ in range(a.warmup):
+        sched.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        sched.step()
+        assert len(sched.last_plan.items) == a.batch and sched.last_plan.n_tokens == a.batch
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    sched.run()
+    return a.batch * a.steps / dt
+
+
+def scheduler_workload(a, cfg, cfg_full, tensors, heads, page, say):
+    """Whole requests through the scheduler: `serve` and `mixed` (see the top of the file)."""
+    import random
+
+    import torch
+
+    from tiny_inference_server_amd.engine import Engine
+    from tiny_inference_server_amd.engine.scheduler import Request, Scheduler
+    from tiny_inference_server_amd.sampling.params import SamplingParams
+    dev = "cuda:0"
+    rng = random.Random(a.seed)
+    gen = torch.Generator().manual_seed(a.seed)
+    elem = 2 if a.dtype == "bfloat16" else 4
+    dkey = "bf16" if a.dtype == "bfloat16" else "fp32"
+    n_req, portion = a.requests, a.prefill_tokens
+    context = min(cfg.max_context, 8192)
+
+    def ids_of(n):
+        return torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
+
+    if a.workload == "serve":
+        new = a.new_tokens
+        longest = min(4096, context - new - 1)
+        lens = [rng.randint(min(128, longest), longest) for _ in range(n_req)]
+        pool = sum(-(-(n + new) // page) * page for n in lens)
+        extra_slots = 0
+    else:
+        # a request whose prompt is in decodes while the others' prompts are still fed: room for those tokens too
+        new = a.steps + a.warmup + 8 + n_req * (context // portion + 1)
+        if new + 2 > context:
+            raise ValueError(f"a context of {context} has no room for {new} decoded tokens")
+        lens = [rng.randint(min(512, context - new - 1), context - new - 1) for _ in range(n_req)]
+        pool = sum(-(-(n + new) // page) * page for n in lens) + 2 * context
+        extra_slots = 1
+    engine = Engine(config=cfg, tensors=tensors, dtype=a.dtype, page_size=page, max_tokens=pool,
+                    max_requests=n_req + extra_slots, device=dev, run_heads=heads)
+    sched = Scheduler(engine, max_batch=n_req + extra_slots, token_budget=portion + n_req, plan="final",
+                      max_context=context)
+    records = []        # (seconds, tokens, decoding requests, tokens held by the step's requests, attention pairs)
+
+    def timed_step():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        sched.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        items = sched.last_plan.items
+        kv = sum(start + n for _, start, n, _ in items)
+        pairs = sum(n * start + n * (n + 1) / 2 for _, start, n, _ in items)
+        n_dec = sum(1 for r, start, n, _ in items if n == 1 and start >= r.prompt_len)
+        records.append((dt, sum(n for _, _, n, _ in items), n_dec, kv, pairs))
+
+    def params(i, n_new):
+        return SamplingParams(max_new_tokens=n_new, seed=a.seed + i, ignore_eos=True, **SAMPLING)
+
+    if a.workload == "serve":
+        say(f"serve: {n_req} requests, prompts of {min(lens)}..{max(lens)} tokens ({sum(lens)} in all), {new} new each")
+        # a short run of the same kind first: the library's set-up and the first captures are not the workload's
+        for i in range(4):
+            sched.submit(Request(ids_of(min(300 + 40 * i, context // 2)), params(i, 8)))
+        sched.run()
+        sched.finished.clear()
+        for i, n in enumerate(lens):
+            sched.submit(Request(ids_of(n), params(i, new)))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while sched.queue or sched.active:
+            sched.admit()
+            timed_step()
+        wall = time.perf_counter() - t0
+        generated = sum(len(r.out_ids()) for r in sched.finished)
+        assert generated == n_req * new, (generated, n_req * new)
+        value, timed = generated / wall, records
+        dec = [r for r in records if r[2] == r[1]]                 # steps of decoded tokens only
+        detail = {"wall_s": round(wall, 3), "steps": len(records), "decode_only_steps": len(dec),
+                  "decode_only_ms": round(1e3 * sum(r[0] for r in dec) / max(1, len(dec)), 3),
+                  "prompt_tokens": sum(lens), "generated_tokens": generated, "preemptions": sched.preempts,
+                  "all_tokens_per_s": round((sum(lens) + generated) / wall, 1)}
+    else:
+        say(f"mixed: {n_req} requests decoding at contexts of {min(lens)}..{max(lens)} tokens, "
+            f"{portion}-token portions of further prompts beside them")
+        for i, n in enumerate(lens):
+            sched.submit(Request(ids_of(n), params(i, new)))
+        sched.admit()
+        while any(r.fed < r.prompt_len for r in sched.active):
+            sched.step()
+        records.clear()
+        # from here on a further prompt is always being fed: each takes the free slot, runs its portions beside the
+        # decoded tokens, generates one token and leaves
+        long_prompt = (context - 2) // portion * portion
+        n_steps = a.steps + a.warmup
+        k = 0
+        while len(records) < n_steps:
+            if not sched.queue and len(sched.active) <= n_req:
+                sched.submit(Request(ids_of(long_prompt), params(n_req + k, 1)))
+                k += 1
+            sched.admit()
+            timed_step()
+        timed = [r for r in records[a.warmup:] if r[2] == n_req and r[1] == n_req + portion]
+        if not timed:
+            raise RuntimeError("no step held the decoding requests and a whole portion")
+        seconds = sum(r[0] for r in timed)
+        value = n_req * len(timed) / seconds
+        detail = {"timed_steps": len(timed), "ms_per_mixed_step": round(1e3 * seconds / len(timed), 3),
+                  "portion_tokens_per_s": round(portion * len(timed) / seconds, 1),
+                  "mean_context": round(sum(lens) / n_req, 1)}
+    floors = [step_floor(cfg, heads, elem, r[1], r[3], r[4], dkey) for r in timed]
+    floor_s, meas_s = sum(f[0] for f in floors), sum(r[0] for r in timed)
+    byts, flops = sum(f[1] for f in floors), sum(f[2] for f in floors)
+    line = {
+        "metric": f"generated tok/s, workload {a.workload} ({a.size}, {dkey}, {n_req} requests through the scheduler)",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": len(timed), "warmup": a.warmup,
+        "ms_per_step": round(1e3 * meas_s / len(timed), 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dkey, "data": "synthetic: random weights N(0,0.02), uniform random token ids",
+        "config": {
+            "model": a.size, "workload": a.workload, "global_batch": n_req, "seq_len": context,
+            "parallelism": "single-gpu", "n_layers": cfg.n_layers, "n_layers_full": cfg_full.n_layers,
+            "d_model": cfg.d_model, "n_heads": cfg.n_heads, "n_kv_heads": cfg.n_kv_heads, "head_dim": cfg.head_dim,
+            "ffn_hidden": cfg.ffn_hidden, "vocab_size": cfg.vocab_size, "mtp_heads_run": cfg.mtp_heads if heads else 0,
+            "tie_embeddings": cfg.tie_embeddings, "page_size": page, "token_budget": portion + n_req,
+            "sampling": "temperature 0.9, top-k 50, top-p 0.95, repetition penalty 1.1",
+        },
+        "roofline": {"bound": "hbm or mfma per step", "achieved": round(floor_s / meas_s, 4), "peak": 1.0,
+                     "unit": "sum of step floors / sum of step times", "frac": round(floor_s / meas_s, 4),
+                     "hbm_GBs": round(byts / meas_s / 1e9, 1), "mfma_TFLOPs": round(flops / meas_s / 1e12, 1)},
+        "detail": detail,
+    }
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -67,6 +253,9 @@ def main() -> int:
     ap.add_argument("--no-trunk-point", dest="trunk_point", action="store_false",
                     help="skip the extra decode measurement without the prediction heads")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--workload", choices=["decode", "serve", "mixed"], default="decode")
+    ap.add_argument("--requests", type=int, default=64, help="serve, mixed: requests (decoding at once)")
+    ap.add_argument("--new-tokens", type=int, default=256, help="serve: tokens generated per request")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
@@ -92,9 +281,11 @@ def main() -> int:
     dev = "cuda:0"
     torch.cuda.set_device(0)
     tensors = random_tensors(cfg, a.seed, dtype=a.dtype, device=dev)
+    page = 16
+    if a.workload != "decode":
+        return scheduler_workload(a, cfg, cfg_full, tensors, heads, page, say)
     points = [int(p) for p in a.points.split(",") if p.strip()]
     max_b = max([a.batch] + points)
-    page = 16
     engine = Engine(config=cfg, tensors=tensors, dtype=a.dtype, page_size=page,
                     max_tokens=max_b * (a.context + page), max_requests=max_b, device=dev, run_heads=heads)
     trunk = None
@@ -163,6 +354,10 @@ def main() -> int:
         # the reference's "plain" decode runs no prediction heads; the same here, for comparison with its numbers
         say(f"decode at batch {a.batch} without the prediction heads")
         pts[f"decode_b{a.batch}_trunk_only"] = round(decode_rate(a.batch, a.steps, a.warmup, trunk)[0], 1)
+    # the same decode at the headline batch through the scheduler: admission, planning, sampling with the reference's
+    # options (server.py:515-516), finishing
+    say(f"decode at batch {a.batch} through the scheduler")
+    pts[f"decode_b{a.batch}_scheduler"] = round(scheduler_decode_rate(engine, a, cfg, gen), 1)
     line = {
         "metric": f"decode tok/s at batch {a.batch} ({a.size}, {dkey}); prefill tok/s at {a.prefill_tokens:,} tokens",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,

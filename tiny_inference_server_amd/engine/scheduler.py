@@ -91,6 +91,7 @@ class Scheduler:
         self.peak_running = 0
         self.steps = 0
         self.tokens_run = 0
+        self.last_plan: Optional[StepPlan] = None       # what the latest step ran, for whoever measures steps
 
     # ---- queueing and admission ----------------------------------------------------------------------
     def submit(self, req: Request) -> None:
@@ -190,6 +191,7 @@ class Scheduler:
                                    f"{self.page_size}, the pool has {self.engine.total_pages()}")
             self.preempt()
         self.peak_running = max(self.peak_running, len(self.active))
+        self.last_plan = plan
         if not plan.items:
             return
         entries = []

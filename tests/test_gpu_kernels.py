@@ -407,9 +407,33 @@ def test_rope_and_cache_write_of_pair_ordered_rows(ops_for, n_heads, n_kv, hd, p
             assert torch.equal(pa.cpu(), plane0)
 
 
-@pytest.mark.parametrize("V", [6, 100, 1000, 48000])
-def test_sampling(ops_for, V):
-    ops, ref = ops_for(torch.float32), TorchOps()
+def assert_same_draws(ref, got, logits, temperature, top_k, top_p, pen, u, ctx_t, off, note=None):
+    """The kernel's tokens against the plain sampler's. The draw inverts a cumulative sum in token order, which the
+    kernel adds in 32-bit and the plain sampler in 64-bit: where the uniform number falls within 2e-6 of the whole
+    mass from a token's edge, either neighbour is right, so a token must lie between the plain sampler's draws at
+    u - 2e-6 and u + 2e-6 (the draw is monotone in u); everywhere else that is equality."""
+    want = ref.sample(logits, temperature, top_k, top_p, pen, u, ctx_t, off).tolist()
+    lo = ref.sample(logits, temperature, top_k, top_p, pen, (u - 2e-6).clamp(min=0.0), ctx_t, off).tolist()
+    hi = ref.sample(logits, temperature, top_k, top_p, pen, (u + 2e-6).clamp(max=1.0), ctx_t, off).tolist()
+    got = got.tolist()
+    for r in range(len(got)):
+        assert got[r] == want[r] or lo[r] <= got[r] <= hi[r], (note, r, got[r], want[r], lo[r], hi[r])
+        if lo[r] == hi[r]:
+            assert got[r] == want[r]
+
+
+@pytest.fixture(params=[1, 0], ids=["registers", "general"])
+def sampling_kernel(request, ops_for):
+    """Both sampling kernels: the one that keeps a row in registers, and the general one alone."""
+    ops = ops_for(torch.float32)
+    ops.sampling.cdll.tis_sample_use_registers(request.param)
+    yield ops
+    ops.sampling.cdll.tis_sample_use_registers(1)
+
+
+@pytest.mark.parametrize("V", [6, 100, 1000, 9001, 48000, 98304, 100003])
+def test_sampling(sampling_kernel, V):
+    ops, ref = sampling_kernel, TorchOps()
     n = 8
     logits = rnd((n, V), torch.float32, 60, 3.0)
     temperature = torch.tensor([0.0, 1.0, 0.8, 1.0, 0.9, 1.3, 1.0, 0.7])
@@ -423,9 +447,27 @@ def test_sampling(ops_for, V):
         u = torch.rand(n, generator=torch.Generator().manual_seed(70 + trial))
         got = ops.sample(logits.cuda(), temperature.cuda(), top_k.cuda(), top_p.cuda(), pen.cuda(), u.cuda(),
                          ctx_t.cuda(), off.cuda()).cpu()
-        want = ref.sample(logits, temperature, top_k, top_p, pen, u, ctx_t, off)
-        assert got.tolist() == want.tolist(), (trial, got.tolist(), want.tolist())
+        assert_same_draws(ref, got, logits, temperature, top_k, top_p, pen, u, ctx_t, off, trial)
     assert ops.argmax(logits.cuda()).cpu().tolist() == logits.argmax(-1).tolist()
+
+
+@pytest.mark.parametrize("V", [300, 48000])
+def test_sampling_with_many_values_at_the_cut(sampling_kernel, V):
+    """All logits equal: every value ties at any top-k cut, so all are kept and the draw is uniform over the
+    vocabulary, token by token in order; a row with a few values above a plateau keeps those and the plateau."""
+    ops, ref = sampling_kernel, TorchOps()
+    n = 6
+    logits = torch.zeros(n, V)
+    logits[3:, :] = -1.0
+    logits[3:, [7, V - 2, V // 2]] = torch.tensor([2.0, 1.0, 1.5])
+    temperature = torch.tensor([1.0, 0.7, 1.0, 1.0, 0.9, 1.0])
+    top_k = torch.tensor([50, 5, 2000 % V, 2, 50, 3], dtype=torch.int32)
+    top_p = torch.zeros(n)           # (with ties a top-p cut is a matter of definition: the kernel keeps all of a tie)
+    pen = torch.ones(n)
+    for trial in range(4):
+        u = torch.rand(n, generator=torch.Generator().manual_seed(170 + trial))
+        got = ops.sample(logits.cuda(), temperature.cuda(), top_k.cuda(), top_p.cuda(), pen.cuda(), u.cuda()).cpu()
+        assert_same_draws(ref, got, logits, temperature, top_k, top_p, pen, u, None, None, trial)
 
 
 def test_sampling_reference_vectors(ops_for):
@@ -547,11 +589,12 @@ def test_skinny_product_with_two_column_tiles_a_workgroup(ops_for, M):
     torch.testing.assert_close(wide[1].double(), x.double() @ w.double().t(), rtol=1e-4, atol=1e-4)
 
 
-def test_sampling_with_the_context_kept_on_the_device(ops_for):
+@pytest.mark.parametrize("V", [777, 48000])
+def test_sampling_with_the_context_kept_on_the_device(sampling_kernel, V):
     """The penalty's context as a byte table per request instead of a token list: same draws, and the kernel marks
     what it drew."""
-    ops = ops_for(torch.float32)
-    n, V = 5, 777
+    ops = sampling_kernel
+    n = 5
     logits = rnd((n, V), torch.float32, 90, 3.0)
     temperature = torch.tensor([0.0, 1.0, 0.8, 1.0, 0.9])
     top_k = torch.tensor([0, 40, 0, 3, 50], dtype=torch.int32)

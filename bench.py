@@ -148,6 +148,7 @@ def scheduler_workload(a, cfg, cfg_full, tensors, heads, page, say):
 
     def timed_step():
         torch.cuda.synchronize()
+        replays = engine.graph_replays
         t0 = time.perf_counter()
         sched.step()
         torch.cuda.synchronize()
@@ -156,7 +157,7 @@ def scheduler_workload(a, cfg, cfg_full, tensors, heads, page, say):
         kv = sum(start + n for _, start, n, _ in items)
         pairs = sum(n * start + n * (n + 1) / 2 for _, start, n, _ in items)
         n_dec = sum(1 for r, start, n, _ in items if n == 1 and start >= r.prompt_len)
-        records.append((dt, sum(n for _, _, n, _ in items), n_dec, kv, pairs))
+        records.append((dt, sum(n for _, _, n, _ in items), n_dec, kv, pairs, engine.graph_replays > replays))
 
     def params(i, n_new):
         return SamplingParams(max_new_tokens=n_new, seed=a.seed + i, ignore_eos=True, **SAMPLING)
@@ -180,8 +181,11 @@ def scheduler_workload(a, cfg, cfg_full, tensors, heads, page, say):
         assert generated == n_req * new, (generated, n_req * new)
         value, timed = generated / wall, records
         dec = [r for r in records if r[2] == r[1]]                 # steps of decoded tokens only
+        eager = [r for r in dec if not r[5]]                       # a shape's first steps: run as they are, or captured
         detail = {"wall_s": round(wall, 3), "steps": len(records), "decode_only_steps": len(dec),
                   "decode_only_ms": round(1e3 * sum(r[0] for r in dec) / max(1, len(dec)), 3),
+                  "decode_only_steps_not_replayed": len(eager),
+                  "decode_only_ms_not_replayed": round(1e3 * sum(r[0] for r in eager) / max(1, len(eager)), 3),
                   "prompt_tokens": sum(lens), "generated_tokens": generated, "preemptions": sched.preempts,
                   "all_tokens_per_s": round((sum(lens) + generated) / wall, 1)}
     else:

@@ -45,6 +45,10 @@ class Request:
     def out_ids(self) -> List[int]:
         return self.ids[self.prompt_len:]
 
+    @property
+    def n_out(self) -> int:
+        return len(self.ids) - self.prompt_len
+
 
 @dataclass
 class StepPlan:
@@ -205,7 +209,7 @@ class Scheduler:
             r.fed += n
         if sampled:
             toks = self.sampler.sample(out.logits, [r.params for r in sampled],
-                                       [len(r.out_ids()) for r in sampled], [r.ids for r in sampled],
+                                       [r.n_out for r in sampled], [r.ids for r in sampled],
                                        slots=[self.engine.requests[r.id][0] for r in sampled],
                                        owners=[(r.id, r.preempted) for r in sampled])
             for r, t in zip(sampled, toks):
@@ -218,12 +222,11 @@ class Scheduler:
         self.active = [r for r in self.active if not r.done]
 
     def finish_check(self, r: Request) -> None:
-        out = r.out_ids()
-        if self.eos >= 0 and not r.params.ignore_eos and self.eos in out:
-            r.ids = r.ids[:r.prompt_len + out.index(self.eos) + 1]
+        """Called after every token appended to r: only the last one can be new."""
+        if self.eos >= 0 and not r.params.ignore_eos and r.n_out > 0 and r.ids[-1] == self.eos:
             r.done = True
-        if len(r.out_ids()) >= r.params.max_new_tokens:
-            r.ids = r.ids[:r.prompt_len + r.params.max_new_tokens]
+        if r.n_out >= r.params.max_new_tokens:
+            del r.ids[r.prompt_len + r.params.max_new_tokens:]
             r.done = True
         if len(r.ids) >= self.max_context:
             r.done = True

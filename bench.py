@@ -229,6 +229,7 @@ def scheduler_workload(a, cfg, cfg_full, tensors, heads, page, say):
             "parallelism": "single-gpu", "n_layers": cfg.n_layers, "n_layers_full": cfg_full.n_layers,
             "d_model": cfg.d_model, "n_heads": cfg.n_heads, "n_kv_heads": cfg.n_kv_heads, "head_dim": cfg.head_dim,
             "ffn_hidden": cfg.ffn_hidden, "vocab_size": cfg.vocab_size, "mtp_heads_run": cfg.mtp_heads if heads else 0,
+            "mtp_head_logits": False,
             "tie_embeddings": cfg.tie_embeddings, "page_size": page, "token_budget": portion + n_req,
             "sampling": "temperature 0.9, top-k 50, top-p 0.95, repetition penalty 1.1",
         },
@@ -375,7 +376,8 @@ def main() -> int:
             "n_layers": cfg.n_layers, "n_layers_full": cfg_full.n_layers, "d_model": cfg.d_model,
             "n_heads": cfg.n_heads, "n_kv_heads": cfg.n_kv_heads, "head_dim": cfg.head_dim,
             "ffn_hidden": cfg.ffn_hidden, "vocab_size": cfg.vocab_size,
-            "mtp_heads_run": cfg.mtp_heads if heads else 0,
+            # the heads' blocks run in every timed step; their logits are not asked for (drafts are not used)
+            "mtp_heads_run": cfg.mtp_heads if heads else 0, "mtp_head_logits": False,
             "tie_embeddings": cfg.tie_embeddings, "rope_base": cfg.rope_base, "page_size": page,
             "sampling": "greedy",
         },

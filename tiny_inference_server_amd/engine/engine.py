@@ -83,7 +83,11 @@ class Engine:
         self._capture_graphs = not getattr(ops, "emulates_graphs", False)
         self.graph_table_pages = 64          # block-table widths are rounded up to this many pages
         self._graphs: "OrderedDict[Tuple[int, int], object]" = OrderedDict()   # least recently used first
-        self.max_graphs = 32                 # each holds its step's activations; the oldest goes when there are more
+        # Each graph holds its step's activations; the least recently used one of its kind goes when there are more.
+        # Steps of single tokens are small and a serving run meets one shape per number of live requests and table
+        # width, so many of them are kept; other steps (prompt portions) hold a portion's activations each.
+        self.max_graphs = 32
+        self.max_decode_graphs = 192
         self._graph_seen: Dict[Tuple[int, int], int] = {}
         self.graph_replays = 0
 
@@ -246,6 +250,13 @@ class Engine:
             head_logits.append(h)
         return lg[0], head_logits, valid[1:]
 
+    def _make_room(self, of_kind, limit: int) -> None:
+        """Drop the least recently used graphs of one kind until another fits under `limit`."""
+        keys = [k for k in self._graphs if of_kind(k)]          # least recently used first
+        while len(keys) >= max(1, limit):
+            self._sync()              # no replay of the graph to be dropped is still running
+            del self._graphs[keys.pop(0)]
+
     def _repeated_step(self, batch_entries):
         """Any other step whose shape has come before: the same requests' row counts, the same places wanted, the
         same work for the attention kernels (a batch of equal prompts, a benchmark's prefill). Returns (logits or
@@ -266,9 +277,7 @@ class Engine:
             self._graph_seen[key] = seen + 1
             if seen < 2:
                 return None, plan
-            if len(self._graphs) >= self.max_graphs:
-                self._sync()
-                self._graphs.popitem(last=False)
+            self._make_room(lambda k: k[0] == "step", self.max_graphs)
             graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size, capture=self._capture_graphs)
         else:
             self._graphs.move_to_end(key)
@@ -304,9 +313,7 @@ class Engine:
                     st.max_kv_len = width * self.page_size
                 outs = self.model.forward(step, self.cache)
                 return self.model.logits(outs[0].hidden, step.stages[0].want_index, len(batch_entries))
-            if len(self._graphs) >= self.max_graphs:
-                self._sync()          # no replay of the graph to be dropped is still running
-                self._graphs.popitem(last=False)
+            self._make_room(lambda k: k[0] != "step", self.max_decode_graphs)
             graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size, occupants,
                                                     capture=self._capture_graphs)
         self.graph_replays += 1

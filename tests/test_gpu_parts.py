@@ -12,7 +12,7 @@ from tiny_inference_server_amd.cache import CacheManager
 from tiny_inference_server_amd.config import ARCHITECTURES, Architecture
 from tiny_inference_server_amd.engine import Engine
 from tiny_inference_server_amd.engine.batch import Entry, build_step_batch
-from tiny_inference_server_amd.parts import (ARRANGEMENTS, MIXERS, CallContext, LayerCall, LayerSpec, ModelSpec, PartSpec,
+from tiny_inference_server_amd.parts import (ARRANGEMENTS, MIXERS, POSITION_ENCODINGS, CallContext, LayerCall, LayerSpec, ModelSpec, PartSpec,
                                              StageSpec, StateNeed, Tensors, build_part, to_compute)
 from tiny_inference_server_amd.weights import random_tensors
 
@@ -471,6 +471,90 @@ def routed_plain(ids, w, cfg, n_experts, stretch):
                                         w[f"l{l}.e{int(choice[r])}.d"]) for r in range(T)])
         x = x + prob[:, None] * y
     return pm.rms_norm(x, w["rms_out.scale"], cfg.rms_eps) @ w["embedding.weight"].T
+
+
+class ToyDistanceBias:
+    """A position encoding that leaves queries and keys alone and lowers a score by slope[h] per position of distance."""
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        return {}
+
+    def __init__(self, spec, tensors, ops):
+        self.ops, self.steepest = ops, float(spec.params["steepest"])
+        self.max_context = int(spec.params["max_context"])
+
+    def rotary(self):
+        return None, False
+
+    def score_slopes(self, n_heads):
+        return (self.steepest * 2.0 ** -torch.arange(n_heads, dtype=torch.float32)).to(self.ops.device)
+
+
+def distance_bias_spec(cfg, steepest):
+    from tiny_inference_server_amd.architectures.gqa_mtp import _block, _norm
+    import dataclasses
+    layers = []
+    for l in range(cfg.n_layers):
+        blk = _block(cfg, f"transformer_block_list.{l}.")
+        pos = PartSpec("position", "toy_distance_bias", {"steepest": steepest, "max_context": cfg.max_context})
+        layers.append(blk.with_part("mixer", dataclasses.replace(blk.part("mixer"),
+                                                                 params={**blk.part("mixer").params, "position": pos})))
+    stage = StageSpec("trunk", 0, PartSpec("stage_input", "token_embedding"), tuple(LayerCall(l) for l in range(cfg.n_layers)),
+                      _norm(cfg, "rms_out.scale"))
+    return ModelSpec(cfg.d_model, cfg.vocab_size, cfg.max_context, tuple(layers), (stage,), "embedding.weight", "embedding.weight")
+
+
+def distance_bias_plain(ids, w, cfg, steepest):
+    T, D, NH, G = len(ids), cfg.d_model, cfg.n_heads, cfg.group_size
+    KVH, hd = NH // G, D // NH
+    x = w["embedding.weight"][torch.tensor(ids)]
+    dist = (torch.arange(T)[None, :] - torch.arange(T)[:, None]).double()          # key position - row position
+    causal = dist <= 0
+    for l in range(cfg.n_layers):
+        pre = f"transformer_block_list.{l}."
+        a = pm.rms_norm(x, w[pre + "att.rms_norm_att.scale"], cfg.rms_eps)
+        q = (a @ w[pre + "att.q_proj.weight"]).view(T, NH, hd)
+        k, v = (a @ w[pre + "att.kv_proj.weight"]).view(T, 2, KVH, hd).unbind(1)
+        heads = []
+        for h in range(NH):
+            s = (q[:, h] @ k[:, h // G].T) * hd ** -0.5 + steepest * 2.0 ** -h * dist
+            heads.append(torch.softmax(s.masked_fill(~causal, float("-inf")), dim=-1) @ v[:, h // G])
+        x = x + torch.stack(heads, dim=1).reshape(T, D) @ w[pre + "att.linear_proj.weight"]
+        f = pm.rms_norm(x, w[pre + "rms_norm_ffn.scale"], cfg.rms_eps)
+        x = x + pm.swiglu_ffn(f, w[pre + "ffn.swig.linear1.weight"], w[pre + "ffn.swig.linear2.weight"], w[pre + "ffn.fc.weight"])
+    return pm.rms_norm(x, w["rms_out.scale"], cfg.rms_eps) @ w["embedding.weight"].T
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_toy_position_encoding_that_works_on_the_scores(dtype, tol):
+    """Not every position encoding rotates: one that adds a bias to the scores, linear in the distance and with a
+    slope per head, is registered from here and runs inside the framework's attention mixer (the general kernel takes
+    such calls). Without the bias the logits would differ by far more than the tolerance (checked)."""
+    from tiny_inference_server_amd.config import GqaMtpConfig
+    POSITION_ENCODINGS.register("toy_distance_bias", ToyDistanceBias, replace=True)
+    steepest = 0.5
+    cfg = GqaMtpConfig(d_model=96, vocab_size=149, max_context=256, rope_base=1e4, n_heads=6, n_layers=2, ffn_hidden=80,
+                       group_size=2, mtp_heads=0, architecture="DistanceBiasToy")
+    ARCHITECTURES.register("DistanceBiasToy", Architecture("DistanceBiasToy", GqaMtpConfig,
+                                                           lambda c: distance_bias_spec(c, steepest)), replace=True)
+    w = random_tensors(cfg, 37, std=0.1, gain_jitter=0.1, dtype="float32")
+    if dtype == "bfloat16":
+        w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    w64 = {k: v.double() for k, v in w.items()}
+    eng = Engine(config=cfg, tensors=w, dtype=dtype, page_size=16, max_tokens=256, max_requests=3)
+    reqs = {"a": H.random_ids(149, 52, 8), "b": H.random_ids(149, 21, 9)}
+    want = {rid: distance_bias_plain(ids, w64, cfg, steepest) for rid, ids in reqs.items()}
+    flat = {rid: distance_bias_plain(ids, w64, cfg, 0.0) for rid, ids in reqs.items()}
+    scale = max(t.abs().max().item() for t in want.values())
+    assert max((want[r] - flat[r]).abs().max().item() for r in reqs) > 20 * tol * scale
+    for trace in (H.whole_trace(reqs), H.mixed_trace(reqs, 2, 5)[0], H.portions_trace({"a": reqs["a"]}, 7)):
+        got, _ = H.run_trace(eng, trace, heads=False)
+        assert got
+        for (rid, p), lg in got.items():
+            assert (lg.double() - want[rid][p]).abs().max() <= tol * max(1.0, scale), (rid, p)
+    ARCHITECTURES.unregister("DistanceBiasToy")
+    POSITION_ENCODINGS.unregister("toy_distance_bias")
 
 
 def test_toy_routed_feed_forward_and_toy_position_encoding_in_the_built_in_block():

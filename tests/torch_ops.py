@@ -120,7 +120,7 @@ class TorchOps:
             plane[:, 1] = vt.reshape(plane.shape[0], n_kv_heads, page_size, head_dim)
 
     # ---- attention over the paged cache -----------------------------------------------------------------
-    def paged_attention(self, q, plane, batch, group, n_heads, n_kv_heads, head_dim, window=0, scale=None):
+    def paged_attention(self, q, plane, batch, group, n_heads, n_kv_heads, head_dim, window=0, scale=None, slopes=None):
         n = q.shape[0]
         page_size = plane.shape[3]
         scale = scale if scale is not None else head_dim ** -0.5
@@ -140,6 +140,8 @@ class TorchOps:
             qr = q[r].float().view(n_heads, head_dim)
             for h in range(n_heads):
                 s = (k[:, h // g] @ qr[h]) * scale
+                if slopes is not None:
+                    s = s + float(slopes[h]) * (js - p).float()
                 out[r, h * head_dim:(h + 1) * head_dim] = torch.softmax(s, dim=0) @ v[:, h // g]
         return out.to(q.dtype)
 

@@ -6,6 +6,8 @@
 // Scores, maximum, sum and the output accumulate in 32-bit (reference paged_attention_kernels.py:86-108);
 // masked keys are never read, so what a reused page still holds cannot reach the result.
 // A page holds a head's keys as [slot][head_dim] and its values as [head_dim][slot].
+// A position encoding that works on the scores brings one slope per query head: the score of key j for the row at
+// position p gets slope[h] * (j - p) added (a bias linear in the distance; null: none).
 // Keys are walked in chunks of a fixed size with a running maximum, so the order of every sum depends on
 // the row's own length only, not on what else is in the batch.
 #include "common.h"
@@ -20,7 +22,7 @@ template <typename T>
 __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     const T* __restrict__ q, long q_ld, const T* __restrict__ plane, const int* __restrict__ block_tables, int bt_ld,
     const int* __restrict__ row_seq, const int* __restrict__ positions, T* __restrict__ out, long out_ld,
-    int group_size, int n_kv_heads, int HD, int page_size, int window, float scale) {
+    int group_size, int n_kv_heads, int HD, int page_size, int window, float scale, const float* __restrict__ slopes) {
   __shared__ float qs[AG_MAX_HD];
   __shared__ float sc[AG_CHUNK];
   __shared__ float red[16];
@@ -34,6 +36,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
   const int* bt = block_tables + (long)row_seq[r] * bt_ld;
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int kv_end = pos + 1;
+  const float slope = slopes ? slopes[h] : 0.f;
 
   for (int d = t; d < HD; d += AG_THREADS) qs[d] = to_f(q[r * q_ld + (long)h * HD + d]) * scale;
   __syncthreads();
@@ -55,6 +58,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
       const T* kp = plane + (long)bt[j / page_size] * page_stride + k_off + (long)(j % page_size) * HD;
       float s = 0.f;
       for (int e = 0; e < HD; ++e) s += qs[e] * to_f(kp[e]);
+      if (slopes) s += slope * (float)(j - pos);
       sc[i] = s;
       cmax = fmaxf(cmax, s);
     }
@@ -92,7 +96,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
 TIS_EXPORT int tis_attention_generic(int dtype, const void* q, long q_ld, const void* plane, const int* block_tables,
                                      int bt_ld, const int* row_seq, const int* positions, void* out, long out_ld,
                                      int rows, int n_heads, int n_kv_heads, int head_dim, int page_size, int window,
-                                     float scale, hipStream_t stream) {
+                                     float scale, const float* slopes, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads || page_size < 1 || window < 0)
     return tis_fail("attention: bad size rows=%d heads=%d kv_heads=%d page=%d window=%d", rows, n_heads, n_kv_heads,
@@ -105,11 +109,11 @@ TIS_EXPORT int tis_attention_generic(int dtype, const void* q, long q_ld, const 
   if (dtype == TIS_F32)
     attention_generic_kernel<float><<<grid, AG_THREADS, 0, stream>>>(
         (const float*)q, q_ld, (const float*)plane, block_tables, bt_ld, row_seq, positions, (float*)out, out_ld, group,
-        n_kv_heads, head_dim, page_size, window, scale);
+        n_kv_heads, head_dim, page_size, window, scale, slopes);
   else if (dtype == TIS_BF16)
     attention_generic_kernel<bf16><<<grid, AG_THREADS, 0, stream>>>(
         (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (bf16*)out, out_ld, group,
-        n_kv_heads, head_dim, page_size, window, scale);
+        n_kv_heads, head_dim, page_size, window, scale, slopes);
   else
     return tis_fail("unknown dtype code %d", dtype);
   return tis_launch_status("attention_generic");

@@ -65,7 +65,7 @@ _SIGNATURES = {
         "tis_rope_write_kv": [_I, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _L, _P],
     }),
     "attention_generic": ("tis_attention_generic", {
-        "tis_attention_generic": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _F, _P],
+        "tis_attention_generic": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _F, _P, _P],
     }),
     "gemm_plain": ("tis_gemm_plain", {
         "tis_gemm_plain": [_I, _I, _P, _L, _P, _L, _P, _L, _P, _L, _I, _I, _I, _P],
@@ -579,10 +579,13 @@ class HipOps:
             raise KernelError(f"cache plane {tuple(plane.shape)} is not [pages, 2, {n_kv_heads}, {page_size}, "
                               f"{head_dim}] contiguous")
 
-    def paged_attention(self, q, plane, batch, group, n_heads, n_kv_heads, head_dim, window=0, scale=None):
+    def paged_attention(self, q, plane, batch, group, n_heads, n_kv_heads, head_dim, window=0, scale=None,
+                        slopes=None):
         """Attention of the rows in `batch` over the cache plane; `q` is [rows, heads*head_dim] (a strided view is fine).
 
-        `batch` brings positions, row_seq and the group's block tables; `group` names the page group.
+        `batch` brings positions, row_seq and the group's block tables; `group` names the page group. `slopes`
+        ([heads] 32-bit, or None): a bias slope[h] * (key position - row position) on the scores; such calls go to
+        the general kernel.
         """
         _rows_view(self._check(q, "q"), "q")
         n = q.shape[0]
@@ -605,7 +608,11 @@ class HipOps:
         if n == 0:
             return out
         group = n_heads // n_kv_heads
-        if (self.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 16 == 0
+        if slopes is not None:
+            self._check(slopes, "score slopes", torch.float32)
+            if slopes.numel() != n_heads or not slopes.is_contiguous():
+                raise KernelError(f"attention: {slopes.numel()} score slopes for {n_heads} heads")
+        if (slopes is None and self.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 16 == 0
                 and group <= 64 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0):
             cols = tile_columns(head_dim)
             plan = batch.extras.get(("attention_items", group, cols, n_kv_heads))
@@ -651,7 +658,7 @@ class HipOps:
         self.attn_generic.tis_attention_generic(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
             _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, head_dim, page_size, int(window),
-            float(scale), self._stream())
+            float(scale), _ptr(slopes), self._stream())
         return out
 
     # ---- sampling ------------------------------------------------------------------------------------

@@ -41,6 +41,9 @@ class GqaAttention:
         self.scale = float(p.get("scale", self.head_dim ** -0.5))
         pos = p["position"]
         self.position = build_part(pos, tensors, ops)
+        # a position encoding may work on the scores instead of (or beside) rotating queries and keys
+        slopes = getattr(self.position, "score_slopes", None)
+        self.slopes = slopes(self.n_heads) if slopes is not None else None
         # one projection for q, k and v: rows of the [out, in] matrix are q heads, then k heads, then v heads.
         # Inside every q and k head the rows are put in pair order (the two members of a rotary pair side by side),
         # so that the kernel that makes them can rotate them while they are still in its registers.
@@ -80,6 +83,7 @@ class GqaAttention:
         page_size = ctx.plane.shape[3]
         q = ops.qkv_rope(x, self.w_qkv, rms, b.positions, b.write_slots[ctx.group], table, ctx.plane, self.n_heads,
                          self.n_kv_heads, self.head_dim, page_size, interleaved, ctx.writes_cache)
+        extra = {"slopes": self.slopes} if self.slopes is not None else {}
         attn = ops.paged_attention(q, ctx.plane, b, ctx.group, self.n_heads, self.n_kv_heads,
-                                   self.head_dim, self.window, self.scale)
+                                   self.head_dim, self.window, self.scale, **extra)
         return ops.linear(attn, self.w_o, residual=residual, reuse_residual=ctx.residual_is_spent)

@@ -13,6 +13,8 @@ every part class
 norm            __call__(x) -> y                       rows in, rows out
 position        rotary() -> (table | None, interleaved)   a table of (cos, sin) per position and pair for
                                                        mixers that rotate queries and keys
+                score_slopes(n_heads) -> [n_heads] | None   optional: a bias slope[h] * (key position - row position)
+                                                       on the attention scores, for encodings that work there
 every part      graph_safe = True                      class attribute, only if what the part launches depends on the
                                                        step's device arrays alone (then decode steps may be captured
                                                        as graphs); absent or False keeps the model on plain launches

@@ -132,7 +132,17 @@ class ToyDecayMixer:
         self.ops, self.decay = ops, float(spec.params["decay"])
         self.w = to_compute(ops, tensors.of(spec, "w").t())
 
+    # a portion's rows are walked on the host; when every request brings one token the state is updated with the step's
+    # device arrays alone, and such steps may be captured as graphs
+    graph_safe = "single_rows"
+
     def forward(self, x, ctx, residual=None):
+        b = ctx.batch
+        if b.max_seq_rows == 1 and b.n_rows == b.n_seqs:
+            slots = b.seq_slots.long()
+            s = self.decay * ctx.state[slots] + x.float()
+            ctx.state[slots] = s
+            return self.ops.linear(s.to(x.dtype), self.w, residual=residual)
         s_all = torch.empty(x.shape[0], x.shape[1], dtype=torch.float32, device=x.device)
         for (first, p0, n), slot in zip(ctx.batch.seq_rows, ctx.batch.host_slots):
             s = ctx.state[slot]
@@ -205,6 +215,15 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
         for (rid, p), lg in got.items():
             want = toy_plain(reqs[rid], w, cfg)[p]
             assert (lg.double() - want).abs().max() <= 2e-5 * max(1.0, want.abs().max()), (rid, p)
+    # the mixer promises graph safety for steps of single tokens only: those are captured and replayed, with the
+    # state living in the request's slot between replays, and portions run as plain launches
+    assert eng.use_decode_graphs and not eng.use_graphs
+    replays = eng.graph_replays
+    got, _ = H.run_trace(eng, H.tail_decode_trace(reqs, 8), heads=False)
+    assert eng.graph_replays >= replays + 5
+    for (rid, p), lg in got.items():
+        want = toy_plain(reqs[rid], w, cfg)[p]
+        assert (lg.double() - want).abs().max() <= 2e-5 * max(1.0, want.abs().max()), (rid, p)
     ARCHITECTURES.unregister("ToyStateModel")
     MIXERS.unregister("toy_decay")
 
@@ -571,7 +590,7 @@ def test_toy_routed_feed_forward_and_toy_position_encoding_in_the_built_in_block
                            replace=True)
     w = random_tensors(cfg, 31, std=0.1, gain_jitter=0.1, dtype="float32")
     eng = Engine(config=cfg, tensors=w, dtype="float32", page_size=16, max_tokens=256, max_requests=3)
-    assert not eng.use_graphs                       # the routed part made no promise about graph capture
+    assert not eng.use_graphs and not eng.use_decode_graphs      # the routed part made no promise about graph capture
     w64 = {k: v.double() for k, v in w.items()}
     reqs = {"a": H.random_ids(157, 45, 3), "b": H.random_ids(157, 18, 4)}
     used = set()

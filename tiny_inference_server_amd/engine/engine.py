@@ -77,7 +77,9 @@ class Engine:
         self._admissions = 0
         self._slot_admission: Dict[int, int] = {}
         # decode steps are replayed from captured graphs where the kernels allow it
-        self.use_graphs = bool(use_graphs) and bool(getattr(ops, "supports_graphs", False)) and self.model.graph_safe
+        can = bool(use_graphs) and bool(getattr(ops, "supports_graphs", False))
+        self.use_graphs = can and self.model.graph_safe                          # any step whose shape repeats
+        self.use_decode_graphs = can and self.model.graph_safe_single_rows       # steps of single tokens
         # an operations object without a device to capture on (a test's stand-in) may ask for the same host logic
         # with plain launches in place of replays
         self._capture_graphs = not getattr(ops, "emulates_graphs", False)
@@ -187,10 +189,10 @@ class Engine:
             self.cache.grow(slot, fed + len(toks))
             batch_entries.append(Entry(slot, fed, arrays[rid], list(want)))
         logits = plan = None
-        if self.use_graphs and not heads:
+        if self.use_decode_graphs and not heads:
             if all(len(e.tokens) == 1 and e.start >= self.model.max_lag and list(e.want) == [0] for e in batch_entries):
                 logits = self._decode_step(batch_entries)
-            else:
+            elif self.use_graphs:
                 logits, plan = self._repeated_step(batch_entries)
         if logits is None:
             if plan is not None:

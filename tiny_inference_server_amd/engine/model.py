@@ -35,7 +35,10 @@ class Model:
         for blk in self.layers:
             # an arrangement that builds no parts of its own answers for itself
             parts += list(getattr(blk, "parts", {}).values()) or [blk]
-        self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
+        # (a part may promise it for steps of single rows only, "single_rows": a recurrence that walks a portion's rows
+        # on the host, but updates its state with device arrays alone when every request brings one token)
+        self.graph_safe = all(getattr(p, "graph_safe", False) is True for p in parts)
+        self.graph_safe_single_rows = all(getattr(p, "graph_safe", False) in (True, "single_rows") for p in parts)
         # host planning that parts ask for, once per distinct key (layers of one shape share a plan)
         self._planners = {}
         for p in parts:

@@ -17,7 +17,9 @@ position        rotary() -> (table | None, interleaved)   a table of (cos, sin) 
                                                        on the attention scores, for encodings that work there
 every part      graph_safe = True                      class attribute, only if what the part launches depends on the
                                                        step's device arrays alone (then decode steps may be captured
-                                                       as graphs); absent or False keeps the model on plain launches
+                                                       as graphs); absent or False keeps the model on plain launches;
+                                                       "single_rows": the promise holds for steps in which every
+                                                       request brings one token (those are still captured)
 mixer           cache_need(params) -> PagedKvNeed | StateNeed | None      classmethod
                 forward(x, ctx, residual=None) -> y    x: normed rows; ctx: CallContext; adds `residual` if given
 feed-forward    forward(x, residual=None) -> y

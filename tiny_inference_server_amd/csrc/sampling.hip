@@ -380,25 +380,38 @@ __global__ __launch_bounds__(SM_THREADS) void sample_regs_kernel(
     in_work = true;
   }
 
-  // keys of the row's values (0 past the end of the row: below every cut that is ever tried), maximum and its index
+  // keys of the row's values (0 past the end of the row: below every cut that is ever tried), maximum and its index.
+  // The values come in batches of CH: all of a batch's loads (logits, and the context's marks where a penalty is
+  // on) are issued before any is used, so a batch costs one trip to memory and not one per value.
+  constexpr int CH = REG % 16 == 0 ? 16 : 8;
+  static_assert(REG % CH == 0, "values per thread come in whole batches");
+  const bool by_mark = pen != 1.f && mark != nullptr;
+  const float* src = by_list ? x : lg;
   unsigned key[REG];
   float mv = -INFINITY;
   int mi = 0x7fffffff;
 #pragma unroll
-  for (int j = 0; j < REG; ++j) {
-    const int i = t + j * SM_THREADS;
-    key[j] = 0u;
-    if (i < V) {
-      float v;
-      if (by_list) {
-        v = x[i];
-      } else {
-        const float l = lg[i];
-        v = l * inv_t;
-        if (pen != 1.f && mark && mark[i]) v = (l > 0.f ? l / pen : l * pen) * inv_t;
-      }
-      key[j] = order_key(v);
-      if (v > mv) { mv = v; mi = i; }
+  for (int c = 0; c < REG; c += CH) {
+    float lv[CH];
+    unsigned char mk[CH];
+#pragma unroll
+    for (int jj = 0; jj < CH; ++jj) {
+      const int i = t + (c + jj) * SM_THREADS;
+      lv[jj] = i < V ? src[i] : 0.f;
+    }
+#pragma unroll
+    for (int jj = 0; jj < CH; ++jj) {
+      const int i = t + (c + jj) * SM_THREADS;
+      mk[jj] = (by_mark && i < V) ? mark[i] : (unsigned char)0;
+    }
+#pragma unroll
+    for (int jj = 0; jj < CH; ++jj) {
+      const int i = t + (c + jj) * SM_THREADS;
+      const float l = lv[jj];
+      float v = by_list ? l : l * inv_t;
+      if (mk[jj]) v = (l > 0.f ? l / pen : l * pen) * inv_t;
+      key[c + jj] = i < V ? order_key(v) : 0u;
+      if (i < V && v > mv) { mv = v; mi = i; }
     }
   }
   block_argmax(mv, mi, sh.sv, sh.si);
@@ -419,16 +432,23 @@ __global__ __launch_bounds__(SM_THREADS) void sample_regs_kernel(
     unsigned pc = 0u;
     int n_cut = V;
     const int wave = t / TIS_WAVE, lane = t % TIS_WAVE;
+    const unsigned kmax = order_key(mv);      // no key of a number lies above it: such candidates need no count
+    int turn = 0;                             // which of the two count buffers the next counted candidate uses
     for (int bit = 31; bit >= 0; --bit) {
       const unsigned cand = pc | (1u << bit);
+      if (cand > kmax) continue;
+      turn ^= 1;
       int c = 0;
 #pragma unroll
-      for (int j = 0; j < REG; ++j) c += __popcll(__ballot(key[j] >= cand));
-      if (lane == 0) sh.counts[bit & 1][wave] = c;
+      for (int j = 0; j < REG; ++j) {
+        c += __popcll(__ballot(key[j] >= cand));
+        if (j % 8 == 7) __builtin_amdgcn_sched_barrier(0);      // eight ballots in scalar registers at a time
+      }
+      if (lane == 0) sh.counts[turn][wave] = c;
       __syncthreads();
       int total = 0;
 #pragma unroll
-      for (int w = 0; w < SM_THREADS / TIS_WAVE; ++w) total += sh.counts[bit & 1][w];
+      for (int w = 0; w < SM_THREADS / TIS_WAVE; ++w) total += sh.counts[turn][w];
       if (total >= k_req) { pc = cand; n_cut = total; }
       if (total == k_req) break;        // exactly k keys reach the candidate: the same set as at the k-th key itself
     }

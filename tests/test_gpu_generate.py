@@ -146,3 +146,31 @@ def test_replay_program(tmp_path, dtype, tol):
                 row += 1
             fed[e["id"]] += len(e["tokens"])
     assert worst <= tol * scale
+
+
+@pytest.mark.parametrize("args,keys", [
+    (["--context", "200", "--steps", "4", "--warmup", "2", "--points", "1", "--prefill-tokens", "64"],
+     ("prefill", "roofline", "points")),
+    (["--workload", "serve", "--requests", "6", "--new-tokens", "5", "--prefill-tokens", "64"], ("roofline", "detail")),
+    (["--workload", "mixed", "--requests", "3", "--steps", "6", "--warmup", "2", "--prefill-tokens", "64"],
+     ("roofline", "detail")),
+])
+def test_bench_modes_run_at_the_tiny_size(args, keys):
+    """bench.py's decode line and its two scheduler workloads, at the tiny preset: one JSON line each, with the
+    contract's fields, a flat `config` of at most 20 keys, and for more than one GPU a refusal with exit code 2."""
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--size", "tiny"] + args,
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    lines = [l for l in proc.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+              "vs_baseline", "dtype", "data", "config") + keys:
+        assert k in d, k
+    assert d["value"] > 0 and d["n_gpus"] == 1 and d["unit"] == "tok/s"
+    assert len(d["config"]) <= 20 and all(not isinstance(v, (dict, list)) for v in d["config"].values())
+    if "points" in keys:
+        assert d["points"]["decode_b1"] > 0 and d["points"]["decode_b8_scheduler"] > 0
+    refused = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True,
+                             text=True, timeout=60)
+    assert refused.returncode == 2 and len(refused.stdout.strip().splitlines()) == 1

@@ -15,7 +15,8 @@ import numpy as np
 import pytest
 
 from tiny_inference_server_amd.ops import hip_ops
-from tiny_inference_server_amd.ops.hip_ops import attention_items, attention_launch_plan, tile_columns
+from tiny_inference_server_amd.ops.hip_ops import (attention_items, attention_launch_plan, decode_items, tile_columns,
+                                                   uneven_lengths)
 
 PRESETS = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tiny_inference_server_amd",
                        "config", "presets")
@@ -48,6 +49,8 @@ CASES = {
     "decode b8 ctx 4096": [(4080 + i, 1) for i in range(8)],
     "decode b64 ctx 4096": [(4032 + i, 1) for i in range(64)],
     "decode b64 ctx 8192": [(8128 + i, 1) for i in range(64)],
+    "decode b64 of uneven lengths": [(17 + 127 * i, 1) for i in range(64)],
+    "decode b5, one long": [(8000, 1), (3, 1), (40, 1), (700, 1), (0, 1)],
     "prompt 512 beside 8 decoding": [(4000 + i, 1) for i in range(8)] + [(1000, 512)],
     "4 prompts of 512": [(0, 512)] * 4,
     "prompt 31 behind 100": [(100, 31)],
@@ -137,6 +140,26 @@ def test_attention_kernels_stay_inside_their_buffers(size, case):
     assert all(cnt * group <= 16 * nb for _, cnt in items)
     assert all(cnt <= TW * (tile_columns(HD) // group) for _, cnt in tiles)
     single = all(r <= 1 for _, _, r in seq_rows)
+    if uneven_lengths(seq_rows):
+        # single rows of very different lengths: the list planned row by row, one entry per wave
+        entries, most = decode_items(seq_rows, nh, kvh, HD)
+        lp = attention_launch_plan(n, len(entries), 0, (0, 0), False, max_kv, nh, kvh, HD, planned_splits=most)
+        assert lp.min_steps == -1 and lp.n_splits == lp.stride == most
+        assert lp.need_floats == lp.row_splits_offset + n <= hip_ops._ATTN_WORKSPACE_FLOATS or lp.stride == 1
+        for row, packed, p, line in entries[entries[:, 0] >= 0].tolist():
+            split, splits = packed & 0xffff, packed >> 16
+            assert 0 <= row < n and p == int(positions[row]) and 0 <= line < len(seq_rows) and split < splits <= most
+            n_steps = (p + 1 + 31) // 32
+            per = -(-n_steps // splits)
+            s_begin, s_end = split * per, min(n_steps, split * per + per)
+            for st in range(s_begin, s_end + 4):
+                for t in range(2):
+                    key0 = st * 32 + t * 16
+                    if st < s_end and key0 < p + 1:
+                        assert key0 >> 4 < table_width
+            slot = (row * nh + nh - 1) * lp.stride + split
+            assert (slot + 1) * HD <= lp.ml_offset or lp.stride == 1
+        return
     for kv_capacity in (max_kv, -(-table_width // 64) * 64 * PAGE):      # eager, and as a captured step sees it
         lp = attention_launch_plan(n, len(items), len(tiles), tile_steps, single, kv_capacity, nh, kvh, HD)
         # workspace: outputs, (maximum, sum) pairs and per-row counts lie one after the other inside it

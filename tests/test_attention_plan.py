@@ -43,3 +43,42 @@ def test_longest_first():
     keys = [first for first, _ in tiles]
     assert keys == sorted(keys, reverse=True)         # a prompt's last rows see the most keys
     assert tuple(items[0]) == (1000, 1)               # the row deep into its request before the short portion
+
+
+def test_decode_items_cover_every_step_once_in_waves_of_even_length():
+    """Single rows of requests that differ widely in length: the planned list gives each row splits by its own
+    length, every entry names its row's position and table line, the list's length depends on the number of rows
+    alone, and no wave walks more than about an even share of all keys."""
+    import random
+    from tiny_inference_server_amd.ops.hip_ops import (decode_items, decode_items_capacity, decode_items_most_splits,
+                                                       uneven_lengths)
+    rng = random.Random(5)
+    for n, kvh, heads, hd in [(64, 3, 12, 128), (5, 4, 16, 128), (17, 8, 32, 128), (2, 1, 3, 48), (300, 2, 4, 64)]:
+        for trial in range(20):
+            pos = [rng.choice([0, 3, 31, 32, 700, 4095, 8000]) if rng.random() < 0.5 else rng.randrange(8192)
+                   for _ in range(n)]
+            seq_rows = [(k + 100, p, 1) for k, p in enumerate(pos)]          # rows of the stage need not start at 0
+            entries, most = decode_items(seq_rows, heads, kvh, hd)
+            assert entries.shape == (decode_items_capacity(n, kvh), 4)
+            assert most == decode_items_most_splits(n, heads, hd) >= 1
+            live = entries[entries[:, 0] >= 0]
+            assert (entries[len(live):, 0] == -1).all()                     # padding only at the end
+            per_row = {}
+            for row, packed, p, line in live.tolist():
+                split, splits = packed & 0xffff, packed >> 16
+                assert p == pos[line] and row == line + 100 and 0 <= split < splits <= most
+                per_row.setdefault(line, []).append((split, splits))
+            assert sorted(per_row) == list(range(n))
+            steps = [(p + 32) // 32 for p in pos]
+            longest = 0
+            for line, got in per_row.items():
+                splits = got[0][1]
+                assert sorted(s for s, _ in got) == list(range(splits)) and splits <= steps[line]
+                longest = max(longest, -(-steps[line] // splits))
+            even = max(4, -(-sum(steps) * kvh // 512))
+            # (a row may not be cut below the fewest steps of a split, nor into more splits than the workspace holds)
+            bound = max(2 * even, max(-(-s // most) for s in steps))
+            assert longest <= bound, (longest, even, most)
+    assert not uneven_lengths([(0, 100, 1), (1, 120, 1), (2, 90, 1)])
+    assert uneven_lengths([(0, 100, 1), (1, 4000, 1), (2, 90, 1)])
+    assert not uneven_lengths([(0, 100, 2), (2, 4000, 1)]) and not uneven_lengths([(0, 4000, 1)])

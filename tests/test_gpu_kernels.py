@@ -148,6 +148,9 @@ def dense_reference(q, k, v, group, pos, window=0):
     (3, 1, 32, 8, [1, 9, 24, 40]),
     (6, 3, 48, 16, [16, 17, 300]),
     (12, 3, 128, 16, [4096, 130]),
+    # lengths that differ a hundredfold in one step: every request gets splits by its own length
+    (12, 3, 128, 16, [1, 5000, 17, 900, 33, 4096, 64, 2, 8100, 640, 31, 32]),
+    (16, 4, 128, 16, [40 + 127 * i for i in range(64)]),
     (5, 5, 8, 4, [3, 1100]),
     (4, 1, 256, 32, [65]),
 ])

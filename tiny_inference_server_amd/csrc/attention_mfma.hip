@@ -72,13 +72,31 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits, int min_steps,
     int split_stride, int* __restrict__ row_splits) {
   const int page_size = PS16 ? 16 : page_size_arg;
-  const int item = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  const int item = blockIdx.x, kvh = blockIdx.y;
+  int split = blockIdx.z;
   const int lane = threadIdx.x, c16 = lane & 15, g = lane >> 4;
-  // no item list: every item is the single row of its own index (a step of decoded tokens), which saves the wave
-  // one of the dependent loads it starts with
-  const int row0 = items ? items[item].x : item, n_rows = items ? items[item].y : 1;
-  const int* bt = block_tables + (long)row_seq[row0] * bt_ld;
-  const int p_first = positions[row0];
+  // Three ways to an item. No item list: every item is the single row of its own index (a step of decoded tokens),
+  // which saves the wave one of the dependent loads it starts with. A list of (first row, rows). Or, for decoded
+  // tokens of requests whose lengths differ widely (min_steps < 0), a list planned on the host with one entry per
+  // wave: (row, split + 65536 * the row's splits, position, line of the block table); it brings what the wave would
+  // otherwise load next, so it costs no further trip to memory, and a row < 0 pads the list to its fixed length.
+  int row0, n_rows, p_first, seq, planned_splits = 0;
+  if (min_steps < 0) {
+    const int4 e = reinterpret_cast<const int4*>(items)[item];
+    if (e.x < 0) return;
+    row0 = e.x;
+    n_rows = 1;
+    split = e.y & 0xffff;
+    planned_splits = e.y >> 16;
+    p_first = e.z;
+    seq = e.w;
+  } else {
+    row0 = items ? items[item].x : item;
+    n_rows = items ? items[item].y : 1;
+    seq = row_seq[row0];
+    p_first = positions[row0];
+  }
+  const int* bt = block_tables + (long)seq * bt_ld;
   const int p_last = p_first + n_rows - 1;
 
   // the lane's column in each block
@@ -119,6 +137,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
   // row_splits tells the merge how many partial results each row has (one: the output is already final).
   int item_splits = n_splits;
   if (min_steps > 0) item_splits = max(1, min(n_splits, n_steps / min_steps));
+  if (min_steps < 0) item_splits = max(1, min(n_splits, planned_splits));
   if (split >= item_splits) return;
   if (row_splits && kvh == 0 && split == 0 && lane < n_rows) row_splits[row0 + lane] = item_splits;
   const int per_split = (n_steps + item_splits - 1) / item_splits;
@@ -835,6 +854,9 @@ TIS_EXPORT int tis_attention_mfma_tile_columns() { return 16 * TNB; }
 // one, [rows][heads][S][HD] floats and [rows][heads][S] float pairs, S the larger of the two. min_steps > 0: an item
 // uses min(n_splits, its steps of 32 keys / min_steps) splits; a tile uses as many as keep each at most
 // tile_max_steps long; row_splits [rows] receives each row's count.
+// min_steps == -1: `items` holds n_items entries of four integers, one per wave and key/value head, planned on the
+// host for single rows: (row, split + 65536 * splits of the row, position, block-table line), row < 0 for padding;
+// n_splits is then the most splits any row may have (the partial results' stride).
 static int attention_launch(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
                             const int* row_seq, const int* positions, const int* items, int n_items, int nb,
                             const int* tiles, int n_tiles, void* out, long out_ld, float* part_o,
@@ -862,7 +884,9 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
     return tis_fail("attention_mfma: bad grid %d x %d (tiles: %d)", n_kv_heads, n_splits, tile_splits);
   const int stride = n_splits > tile_splits ? n_splits : tile_splits;
   if (stride > 1 && (!part_o || !part_ml)) return tis_fail("attention_mfma: %d splits need a workspace", stride);
-  if (min_steps < 0 || (min_steps > 0 && n_splits > 1 && !row_splits))
+  if (min_steps < -1 || (min_steps == -1 && (!items || n_items < 1 || n_tiles > 0)))
+    return tis_fail("attention_mfma: min_steps=%d; -1 goes with a planned list of single rows and no tiles", min_steps);
+  if (min_steps != 0 && n_splits > 1 && !row_splits)
     return tis_fail("attention_mfma: splits chosen item by item (min_steps=%d) need the per-row count array", min_steps);
   if (n_tiles > 0 && tile_max_steps < 1) return tis_fail("attention_mfma: a tile's splits need a longest chain of at least one step");
   if (n_tiles > 0 && stride > 1 && (!row_splits || (n_items > 0 && min_steps < 1)))
@@ -873,7 +897,7 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
   const float scale_log2 = scale * 1.4426950408889634f;
   int rc = 0;
   if (n_items > 0) {
-    dim3 grid(n_items, n_kv_heads, n_splits);
+    dim3 grid(n_items, n_kv_heads, min_steps < 0 ? 1 : n_splits);
 #define LAUNCH(NBV, PSV)                                                                                              \
   attention_mfma_kernel<NBV, PSV><<<grid, 64, 0, stream>>>(                                                      \
       (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)items,     \

@@ -121,14 +121,24 @@ class StepPlan:
 
 
 def build_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: Sequence[bool], cache, device,
-                     max_context: int, plan_rows=None) -> StepBatch:
+                     max_context: int, plan_rows=None, mode=None) -> StepBatch:
     """Row arrays for every stage of one step. `cache` is the CacheManager that already covers the new positions."""
-    return materialize(plan_step_batch(entries, lags, has_source, cache, max_context, plan_rows), device)
+    return materialize(plan_step_batch(entries, lags, has_source, cache, max_context, plan_rows, mode=mode), device)
+
+
+def first_stage_rows(entries: Sequence[Entry]) -> List[Tuple[int, int, int]]:
+    """(first row, first position, rows) per entry, as the first stage (lag 0) sees the step."""
+    out, first = [], 0
+    for e in entries:
+        out.append((first, e.start, len(e.tokens)))
+        first += len(e.tokens)
+    return out
 
 
 def plan_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: Sequence[bool], cache,
-                    max_context: int, plan_rows=None, table_width: Optional[int] = None) -> StepPlan:
-    """The host half: every array of the step, packed. `table_width` pads the block tables to a fixed width."""
+                    max_context: int, plan_rows=None, table_width: Optional[int] = None, mode=None) -> StepPlan:
+    """The host half: every array of the step, packed. `table_width` pads the block tables to a fixed width; `mode`
+    is what the model's plan_mode said about the step and goes back to plan_rows with every stage's rows."""
     n_seqs = len(entries)
     pk = _Packer()
     page_size = cache.page_size
@@ -205,7 +215,9 @@ def plan_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: S
                 ok = p >= p0 and n > 0
                 want.append(first_row + (p - p0) if ok else -1)
                 valid.append(ok)
-        extra = plan_rows(seq_rows, pk.add) if plan_rows is not None else {}
+        extra = {}
+        if plan_rows is not None:
+            extra = plan_rows(seq_rows, pk.add, mode) if mode is not None else plan_rows(seq_rows, pk.add)
         plans.append(dict(
             extra=extra, lag=lag, n_rows=n_rows, tokens=pk.add(tokens), positions=pk.add(positions),
             row_seq=pk.add(row_seq), cu=pk.add(cu), ws=ws,

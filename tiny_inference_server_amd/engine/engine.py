@@ -18,7 +18,7 @@ from .. import architectures  # noqa: F401  (registers the built-in architecture
 from ..cache.manager import CacheManager, OutOfPages
 from ..config.model_config import ARCHITECTURES, load_config
 from ..weights.loader import load_tensors
-from .batch import Entry, build_step_batch, materialize, plan_step_batch
+from .batch import Entry, build_step_batch, first_stage_rows, materialize, plan_step_batch
 from .model import Model
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
@@ -91,6 +91,7 @@ class Engine:
         self.max_graphs = 32
         self.max_decode_graphs = 192
         self._graph_seen: Dict[Tuple[int, int], int] = {}
+        self._has_windows = any(g.spec.window > 0 for g in self.cache.groups.values())
         self.graph_replays = 0
 
     # ---- requests ------------------------------------------------------------------------------------
@@ -149,6 +150,39 @@ class Engine:
         """
         if not entries:
             raise ValueError("a step needs at least one entry")
+        batch_entries = self._single_token_entries(entries)
+        if batch_entries is None:
+            batch_entries = self._checked_entries(entries)
+        return self._run(entries, batch_entries, heads)
+
+    def _single_token_entries(self, entries):
+        """The step that serving is mostly made of: one token for each of some live requests. Returns its batch
+        entries, pages taken, or None for any other step and for whatever is wrong with this one (the general path
+        then says what). A request can only need a page when its next position opens one, so nothing is asked of the
+        cache for the other fifteen of sixteen."""
+        reqs, vocab, ctx, ps = self.requests, self.spec.vocab_size, self.spec.max_context, self.page_size
+        out, opening, slots = [], {}, set()
+        for rid, toks, want in entries:
+            info = reqs.get(rid)
+            if info is None or len(toks) != 1:
+                return None
+            t = toks[0]
+            slot, fed = info
+            if not isinstance(t, (int, np.integer)) or not (0 <= t < vocab) or fed >= ctx or slot in slots:
+                return None
+            slots.add(slot)
+            if fed % ps == 0:
+                opening[slot] = fed + 1
+            out.append(Entry(slot, fed, [int(t)], list(want)))
+        if opening:
+            if not self.cache.can_grow(opening):
+                return None
+            for slot, n in opening.items():
+                self.cache.grow(slot, n)
+        return out
+
+    def _checked_entries(self, entries):
+        """Any step: its entries checked, new requests opened, pages taken for all of it or for none of it."""
         seen = set()
         arrays = {}
         for rid, toks, _ in entries:
@@ -188,6 +222,9 @@ class Engine:
             slot, fed = self.requests[rid]
             self.cache.grow(slot, fed + len(toks))
             batch_entries.append(Entry(slot, fed, arrays[rid], list(want)))
+        return batch_entries
+
+    def _run(self, entries, batch_entries, heads):
         logits = plan = None
         if self.use_decode_graphs and not heads:
             if all(len(e.tokens) == 1 and e.start >= self.model.max_lag and list(e.want) == [0] for e in batch_entries):
@@ -199,7 +236,8 @@ class Engine:
                 step = materialize(plan, self.device)
             else:
                 step = build_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
-                                        self.device, self.spec.max_context, self.model.plan_rows)
+                                        self.device, self.spec.max_context, self.model.plan_rows,
+                                        mode=self.model.plan_mode(first_stage_rows(batch_entries)))
             outs = self.model.forward(step, self.cache)
         n = sum(len(e.want) for e in batch_entries)
         head_logits = head_valid = None
@@ -208,10 +246,12 @@ class Engine:
                 logits, head_logits, head_valid = self._all_logits(outs, n)
             else:
                 logits = self.logits_of(outs, step, n)
-        for rid, toks, _ in entries:
-            slot, fed = self.requests[rid]
-            self.requests[rid] = (slot, fed + len(toks))
-            self.cache.release_behind(slot, fed + len(toks), self.model.max_lag)
+        windows = self._has_windows
+        for (rid, _, _), e in zip(entries, batch_entries):
+            fed = e.start + len(e.tokens)
+            self.requests[rid] = (e.slot, fed)
+            if windows:
+                self.cache.release_behind(e.slot, fed, self.model.max_lag)
         return StepOutput(logits, head_logits, head_valid)
 
     def _sync(self):
@@ -267,7 +307,8 @@ class Engine:
         pages = max((max(len(g.tables[e.slot]) for e in batch_entries) for g in self.cache.groups.values()), default=1)
         width = -(-pages // self.graph_table_pages) * self.graph_table_pages
         plan = plan_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
-                               self.spec.max_context, self.model.plan_rows, table_width=width)
+                               self.spec.max_context, self.model.plan_rows, table_width=width,
+                               mode=self.model.plan_mode(first_stage_rows(batch_entries)))
         # what the host decides from, beyond the arrays' shapes
         key = ("step", width, plan.layout(),
                tuple((pl["max_rows"], pl["keep_count"], pl["previous_rows"], tuple(pl["valid"])) for pl in plan.plans))
@@ -291,7 +332,9 @@ class Engine:
         from .graph import DecodeGraph
         pages = max((max(len(g.tables[e.slot]) for e in batch_entries) for g in self.cache.groups.values()), default=1)
         width = -(-pages // self.graph_table_pages) * self.graph_table_pages
-        key = (len(batch_entries), width)
+        # (what the parts' planning says about the step, e.g. requests of very different lengths, changes the launches)
+        mode = self.model.plan_mode(first_stage_rows(batch_entries))
+        key = (len(batch_entries), width, mode)
         graph = self._graphs.get(key)
         if graph is not None:
             self._graphs.move_to_end(key)
@@ -303,7 +346,7 @@ class Engine:
             self.graph_replays += 1
             return graph.run_same_requests(batch_entries)
         plan = plan_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
-                               self.spec.max_context, self.model.plan_rows, table_width=width)
+                               self.spec.max_context, self.model.plan_rows, table_width=width, mode=mode)
         if graph is None:
             seen = self._graph_seen.get(key, 0)
             self._graph_seen[key] = seen + 1
@@ -317,6 +360,6 @@ class Engine:
                 return self.model.logits(outs[0].hidden, step.stages[0].want_index, len(batch_entries))
             self._make_room(lambda k: k[0] != "step", self.max_decode_graphs)
             graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size, occupants,
-                                                    capture=self._capture_graphs)
+                                                    capture=self._capture_graphs, mode=mode)
         self.graph_replays += 1
         return graph.run(plan, occupants)

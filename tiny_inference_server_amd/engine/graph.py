@@ -38,8 +38,9 @@ class DecodeGraph:
     operations object without a device (a test's stand-in) exercises this file's host logic.
     """
 
-    def __init__(self, engine, plan: StepPlan, kv_capacity: int, occupants=None, capture: bool = True):
+    def __init__(self, engine, plan: StepPlan, kv_capacity: int, occupants=None, capture: bool = True, mode=None):
         self.layout = plan.layout()
+        self.mode = mode
         self.engine = engine
         self.capture = capture
         dev = engine.device
@@ -68,6 +69,11 @@ class DecodeGraph:
                               ws={g: off(i) for g, i in pl["ws"].items()}) for pl in plan.plans]
         self.pages_held = {g: np.array([len(engine.cache.groups[g].tables[s]) for s in self.slots])
                            for g in self.table_at}
+        # what the parts planned for each stage (work lists of their kernels): where each array lies, in the order
+        # the planning added them, and the host values that the captured launches were made from
+        self.extras_at = [[(off(i), plan.packer.offsets[i][1]) for i in sorted(v[0] for v in pl["extra"].values())]
+                          for pl in plan.plans]
+        self.extras_host = [tuple(sorted((k, v[1:]) for k, v in pl["extra"].items())) for pl in plan.plans]
 
     def _launch(self):
         engine, n = self.engine, self.step.n_wanted
@@ -111,6 +117,23 @@ class DecodeGraph:
                 t_off, (rows, width) = self.table_at[g]
                 table = flat[t_off:t_off + rows * width].reshape(rows, width)
                 flat[w_off:w_off + n] = table[rows_idx, pos // ps] * ps + pos % ps
+        if any(self.extras_at):
+            # the parts plan again for the new positions, into the places their arrays have in the buffer
+            for at, host_values, st in zip(self.extras_at, self.extras_host, self.stage_at):
+                slots_left = list(at)
+
+                def put(arr, shape=None, slots_left=slots_left):
+                    a = np.ascontiguousarray(arr, dtype=np.int32).reshape(-1)
+                    if not slots_left or int(np.prod(slots_left[0][1])) != a.size:
+                        raise RuntimeError("a part planned an array that the captured step has no place for")
+                    o, _ = slots_left.pop(0)
+                    flat[o:o + a.size] = a
+                    return -1
+
+                pos = starts - st["lag"]
+                extra = self.engine.model.plan_rows([(k, int(pos[k]), 1) for k in range(n)], put, self.mode)
+                if slots_left or tuple(sorted((k, v[1:]) for k, v in extra.items())) != host_values:
+                    raise RuntimeError("the parts' planning no longer fits the captured step")
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
         self._replay()

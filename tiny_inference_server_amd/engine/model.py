@@ -83,11 +83,20 @@ class Model:
     def cache_needs(self) -> Dict[str, object]:
         return dict(self.needs)
 
-    def plan_rows(self, seq_rows, add):
+    def plan_mode(self, seq_rows):
+        """What kind of plans a step gets, decided once from the first stage's rows (first row, first position, rows
+        per request) and handed to plan_rows for every stage: hashable, and part of what must be equal for two steps
+        to share a captured graph. None: nothing to say."""
+        modes = tuple((key, part.plan_mode(seq_rows)) for key, part in self._planners.items() if hasattr(part, "plan_mode"))
+        modes = tuple(m for m in modes if m[1] is not None)
+        return modes or None
+
+    def plan_rows(self, seq_rows, add, mode=None):
         """Host planning of every part that asks for it, for one stage's rows: {name: (packed array id, values...)}."""
         plans = {}
-        for part in self._planners.values():
-            plans.update(part.plan_rows(seq_rows, add))
+        of = dict(mode) if mode else {}
+        for key, part in self._planners.items():
+            plans.update(part.plan_rows(seq_rows, add, of[key]) if key in of else part.plan_rows(seq_rows, add))
         return plans
 
     def _bind(self, ctx, key, cache):

@@ -108,6 +108,13 @@ _ATTN_TARGET_WAVES = 512
 _ATTN_PROMPT_TARGET_WAVES = 2048  # what the grid offers where rows of prompts are in the batch ...
 _ATTN_PROMPT_SPLIT_MAX_ROWS = 512 # ... and the batch is small; a long portion fills the chip by its rows alone
 _ATTN_PROMPT_MIN_STEPS = 8         # steps of 32 keys below which a prompt item's split is not worth its merge
+_ATTN_UNEVEN = 1.5              # decoded tokens: from this ratio of the longest request to the mean on, splits are planned
+                                # request by request on the host instead of being the same for all
+_ATTN_DECODE_MAX_SPLITS = 64    # ... and the most that one request may get
+_ATTN_PLANNED_MAX_WAVES = 192   # ... where requests x key/value heads leave room for three splits each: with fewer
+                                # splits to shift between requests the plain grid was as fast or faster (64 uneven
+                                # requests, planned / same splits, us: 3 kv heads 48 / 58, 4: 72 / 70, 8: 162 / 125;
+                                # 16 requests: 18.5 / 20.8, 21.3 / 22.2, 34.3 / 36.7)
 _ATTN_MIN_SPLIT_KEYS = 128      # a split shorter than this costs more in merging than it gains in spreading
 _ATTN_TILE_WAVES = 4            # waves of the workgroup that takes a tile of a long portion
 _ATTN_TILE_GROUPS = 512         # workgroups of the tile kernel that the chip runs side by side
@@ -187,6 +194,68 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
     return nb, cut(rest, max(1, (16 * nb) // group_size))[0], tiles, steps
 
 
+def uneven_lengths(seq_rows) -> bool:
+    """Whether a step of single rows holds requests of such different lengths that equal split counts would leave the
+    longest request's waves running on alone: then the splits are planned request by request (decode_items)."""
+    n = len(seq_rows)
+    if n < 2:
+        return False
+    longest = total = 0
+    for _, p0, rows in seq_rows:            # (one pass: this runs for every step of decoded tokens)
+        if rows != 1:
+            return False
+        steps = (p0 + 32) >> 5
+        total += steps
+        if steps > longest:
+            longest = steps
+    return longest * n > _ATTN_UNEVEN * total + 2 * n
+
+
+def decode_items_capacity(n_rows: int, n_kv_heads: int) -> int:
+    """Entries of a planned list for `n_rows` single rows: what the splits can add up to, whatever the lengths."""
+    # (a multiple of the eight XCDs: workgroups go to them in turn, so the waves of an entry's key/value heads, which
+    # read the same pages, then meet in one L2: 162 against 183 us at 8 key/value heads)
+    return -(-(_ATTN_TARGET_WAVES // n_kv_heads + n_rows + 1) // 8) * 8
+
+
+def decode_items_most_splits(n_rows: int, n_heads: int, head_dim: int, workspace_floats=None) -> int:
+    """The most splits one row of such a list may have: bounded by the workspace for partial results."""
+    workspace_floats = _ATTN_WORKSPACE_FLOATS if workspace_floats is None else workspace_floats
+    return int(max(1, min(_ATTN_DECODE_MAX_SPLITS, (workspace_floats - n_rows) // (n_rows * n_heads * (head_dim + 2)))))
+
+
+def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspace_floats=None):
+    """The work list of a step of single rows whose requests differ widely in length: one entry per wave (and
+    key/value head), (row, split + 65536 * splits of the row, position, block-table line), so that every wave walks
+    about the same number of keys; longest first; padded with row -1 to a length that depends on the number of rows
+    alone (a captured launch keeps its grid while the lengths change). Returns (int32 [capacity, 4], most splits)."""
+    n = len(seq_rows)
+    rows = np.fromiter((f for f, _, _ in seq_rows), dtype=np.int64, count=n)
+    pos = np.fromiter((p0 for _, p0, _ in seq_rows), dtype=np.int64, count=n)
+    steps = (pos + 32) // 32                                     # a row at position p sees p + 1 keys
+    fewest = max(1, _ATTN_MIN_SPLIT_KEYS // 32)
+    even = max(fewest, -(-int(steps.sum()) * n_kv_heads // _ATTN_TARGET_WAVES))
+    most = decode_items_most_splits(n, n_heads, head_dim, workspace_floats)
+    splits = np.clip((steps + even // 2) // even, 1, np.minimum(steps, most))
+    cap = decode_items_capacity(n, n_kv_heads)
+    total = int(splits.sum())
+    if total > cap:
+        raise KernelError(f"attention: {total} planned splits for a list of {cap}")
+    # one entry per (row, split); those with the most steps first, and among equals split by split over all rows, so
+    # that waves that start together read different requests' pages (the order a grid of rows x splits would have)
+    who = np.repeat(np.arange(n), splits)
+    which = np.arange(total) - np.repeat(np.cumsum(splits) - splits, splits)
+    per_split = -(-steps // splits)
+    by = np.lexsort((who, which, -per_split[who]))
+    who, which = who[by], which[by]
+    out = np.full((cap, 4), -1, dtype=np.int32)
+    out[:total, 0] = rows[who]
+    out[:total, 1] = which + (splits[who] << 16)
+    out[:total, 2] = pos[who]
+    out[:total, 3] = who
+    return out, most
+
+
 class AttentionLaunch(NamedTuple):
     """How one call of the matrix-core attention cuts its keys, and where its partial results lie in the workspace
     (offsets in floats): [rows][heads][stride][head size] outputs, then [rows][heads][stride] (maximum, sum) pairs,
@@ -202,11 +271,14 @@ class AttentionLaunch(NamedTuple):
 
 
 def attention_launch_plan(n, n_items, n_tiles, tile_steps, single, max_kv_len, n_heads, n_kv_heads, head_dim,
-                          workspace_floats=None) -> AttentionLaunch:
-    """Split counts of one attention call over `n` rows, from the planner's items and tiles; pure host arithmetic."""
+                          workspace_floats=None, planned_splits=0) -> AttentionLaunch:
+    """Split counts of one attention call over `n` rows, from the planner's items and tiles; pure host arithmetic.
+    planned_splits > 0: the items are a list planned by decode_items, whose rows have at most that many splits."""
     workspace_floats = _ATTN_WORKSPACE_FLOATS if workspace_floats is None else workspace_floats
     n_splits, min_steps, tile_splits, tile_max_steps = 1, 0, 1, 1 << 20
-    if n_items:
+    if planned_splits:
+        n_splits, min_steps = planned_splits, -1
+    elif n_items:
         # decoded tokens: every request's keys are cut into the same number of splits, enough to spread a
         # short batch over the chip. Prompt rows: the grid offers more splits than the chip needs and every
         # item takes as many as its own length deserves (the kernel decides, from _ATTN_PROMPT_MIN_STEPS),
@@ -279,12 +351,21 @@ class HipOps:
             if dtype == torch.bfloat16 else None
 
     # ---- planning on the host --------------------------------------------------------------------------
-    def plan_attention(self, n_heads: int, n_kv_heads: int, head_dim: int, seq_rows, add):
+    def plan_attention_mode(self, seq_rows):
+        """What kind of plan a step gets, from its first stage's rows: two steps may share a captured graph only if
+        this is equal. "uneven": single rows of requests that differ widely in length."""
+        return "uneven" if self.dtype == torch.bfloat16 and uneven_lengths(seq_rows) else None
+
+    def plan_attention(self, n_heads: int, n_kv_heads: int, head_dim: int, seq_rows, add, mode=None):
         """An attention mixer's host planning, called while a step's arrays are packed: the work items of the
         matrix-core kernels for the step's rows. Returns {name: (packed array id, host values...)}."""
         plans = {}
         if self.dtype == torch.bfloat16:
             group, cols = n_heads // n_kv_heads, tile_columns(head_dim)
+            if (mode == "uneven" and group <= 64 and len(seq_rows) * n_kv_heads <= _ATTN_PLANNED_MAX_WAVES
+                    and all(n == 1 for _, _, n in seq_rows)):
+                entries, most = decode_items(seq_rows, n_heads, n_kv_heads, head_dim)
+                return {("attention_decode_items", group, cols, n_kv_heads): (add(entries), len(entries), most)}
             nb, items, tiles, steps = attention_items(seq_rows, group, cols, n_kv_heads)
             if nb <= 4 and (len(items) or len(tiles)):
                 # one array: the items' lines, then the tiles'
@@ -615,17 +696,35 @@ class HipOps:
         if (slopes is None and self.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 16 == 0
                 and group <= 64 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0):
             cols = tile_columns(head_dim)
+            planned = batch.extras.get(("attention_decode_items", group, cols, n_kv_heads))
             plan = batch.extras.get(("attention_items", group, cols, n_kv_heads))
-            if plan is None:        # a caller that did not plan (a kernel test): plan now, tiles wherever they fit
-                nb, host_items, host_tiles, steps = attention_items(batch.seq_rows, group, cols)
-                both = np.ascontiguousarray(np.concatenate((host_items, host_tiles)))
-                plan = (torch.from_numpy(both).reshape(-1).to(self.device), len(host_items), nb, len(host_tiles), steps)
-            lines, n_items, nb, n_tiles, tile_steps = plan
-            lines = lines.reshape(-1)
-            items = lines[:2 * n_items] if n_items else None
-            tiles = lines[2 * n_items:] if n_tiles else None
-            if batch.max_seq_rows <= 1 and n_items == n:
-                items = None        # single rows in order: the kernel needs no list
+            if planned is None and plan is None:
+                # a caller that did not plan (a kernel test): plan now, tiles wherever they fit
+                if uneven_lengths(batch.seq_rows) and n * n_kv_heads <= _ATTN_PLANNED_MAX_WAVES:
+                    entries, most = decode_items(batch.seq_rows, n_heads, n_kv_heads, head_dim)
+                    planned = (torch.from_numpy(entries).reshape(-1).to(self.device), len(entries), most)
+                else:
+                    nb, host_items, host_tiles, steps = attention_items(batch.seq_rows, group, cols)
+                    both = np.ascontiguousarray(np.concatenate((host_items, host_tiles)))
+                    plan = (torch.from_numpy(both).reshape(-1).to(self.device), len(host_items), nb, len(host_tiles), steps)
+            planned_splits = 0
+            if planned is not None:
+                # single rows with splits planned row by row: one entry of four integers per wave
+                lines, n_items, planned_splits = planned
+                lines = lines.reshape(-1)
+                if batch.max_seq_rows > 1 or lines.numel() != 4 * n_items:
+                    raise KernelError(f"attention: a planned list of {lines.numel()} integers for {n_items} entries "
+                                      f"of single rows ({batch.max_seq_rows} rows a request)")
+                items, tiles, n_tiles, tile_steps, nb = lines, None, 0, (0, 0), 1
+                while group > 16 * nb:
+                    nb *= 2
+            else:
+                lines, n_items, nb, n_tiles, tile_steps = plan
+                lines = lines.reshape(-1)
+                items = lines[:2 * n_items] if n_items else None
+                tiles = lines[2 * n_items:] if n_tiles else None
+                if batch.max_seq_rows <= 1 and n_items == n:
+                    items = None        # single rows in order: the kernel needs no list
             lib = self._attn_mfma.get(head_dim)
             if lib is None:
                 lib = self._attn_mfma[head_dim] = library(f"attention_mfma@{head_dim}")
@@ -635,7 +734,7 @@ class HipOps:
                                       f"assumes {cols}")
             single = items is None and n_tiles == 0
             lp = attention_launch_plan(n, n_items, n_tiles, tile_steps, single, batch.max_kv_len, n_heads, n_kv_heads,
-                                       head_dim)
+                                       head_dim, planned_splits=planned_splits)
             n_splits, min_steps, tile_splits, tile_max_steps = lp.n_splits, lp.min_steps, lp.tile_splits, lp.tile_max_steps
             part_o = part_ml = row_splits = None
             if lp.stride > 1:
@@ -644,9 +743,10 @@ class HipOps:
                                       f"{self._workspace.numel()}")
                 part_o = self._workspace
                 part_ml = self._workspace[lp.ml_offset:]
-                if not single:
+                if lp.min_steps != 0 or n_tiles:
                     row_splits = self._workspace[lp.row_splits_offset:]
-            if lines.numel() < 2 * (n_items + n_tiles) or lines.dtype != torch.int32 or not lines.is_contiguous():
+            if (not planned_splits and lines.numel() < 2 * (n_items + n_tiles)) or lines.dtype != torch.int32 \
+                    or not lines.is_contiguous():
                 raise KernelError(f"attention: the work list holds {lines.numel()} entries for {n_items} items and "
                                   f"{n_tiles} tiles")
             lib.tis_attention_mfma(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0),

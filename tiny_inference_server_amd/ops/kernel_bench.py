@@ -52,7 +52,7 @@ def parse_segments(text: str):
 
 
 def attention_case(ops, a):
-    from .hip_ops import attention_items, tile_columns
+    from .hip_ops import _ATTN_PLANNED_MAX_WAVES, attention_items, decode_items, tile_columns, uneven_lengths
     nh, kvh, hd, ps = a.heads, a.kv_heads, a.head_dim, a.page_size
     segs = parse_segments(a.segments)
     pages = [-(-(p0 + n) // ps) for p0, n in segs]
@@ -72,11 +72,17 @@ def attention_case(ops, a):
                             block_tables={"g": tables.to(ops.device)}, max_kv_len=max(p0 + n for p0, n in segs),
                             extras={}, n_rows=rows, max_seq_rows=max(n for _, n in segs), seq_rows=seq_rows)
     # --no-tiles: what the one-wave kernel alone makes of the same rows; --tiles: tiles however little work there is
-    nb, items, tiles, steps = attention_items(seq_rows, nh // kvh, 0 if a.no_tiles else tile_columns(hd),
-                                              0 if a.tiles else kvh)
     import numpy as np
-    both = torch.from_numpy(np.ascontiguousarray(np.concatenate((items, tiles)))).reshape(-1).to(ops.device)
-    batch.extras[("attention_items", nh // kvh, tile_columns(hd), kvh)] = (both, len(items), nb, len(tiles), steps)
+    if ((uneven_lengths(seq_rows) and len(seq_rows) * kvh <= _ATTN_PLANNED_MAX_WAVES) or a.planned) and not a.same_splits:
+        # decoded tokens of requests that differ widely in length: splits planned request by request, as the engine does
+        entries, most = decode_items(seq_rows, nh, kvh, hd)
+        batch.extras[("attention_decode_items", nh // kvh, tile_columns(hd), kvh)] = (
+            torch.from_numpy(entries).reshape(-1).to(ops.device), len(entries), most)
+    else:
+        nb, items, tiles, steps = attention_items(seq_rows, nh // kvh, 0 if a.no_tiles else tile_columns(hd),
+                                                  0 if a.tiles else kvh)
+        both = torch.from_numpy(np.ascontiguousarray(np.concatenate((items, tiles)))).reshape(-1).to(ops.device)
+        batch.extras[("attention_items", nh // kvh, tile_columns(hd), kvh)] = (both, len(items), nb, len(tiles), steps)
     us = graph_time(lambda: ops.paged_attention(q, plane, batch, "g", nh, kvh, hd), a.reps)
     kv_bytes = sum(p0 + n for p0, n in segs) * kvh * hd * 2 * 2
     flops = sum(4 * nh * hd * (n * p0 + n * (n + 1) / 2) for p0, n in segs)
@@ -110,6 +116,10 @@ def main(argv=None) -> int:
     at.add_argument("--page-size", type=int, default=16)
     at.add_argument("--no-tiles", action="store_true", help="long portions too go to the one-wave kernel")
     at.add_argument("--tiles", action="store_true", help="long portions go to the workgroup kernel however few they are")
+    at.add_argument("--planned", action="store_true",
+                    help="decoded tokens: splits planned request by request also where the lengths are alike")
+    at.add_argument("--same-splits", action="store_true",
+                    help="decoded tokens: every request gets the same number of splits, however their lengths differ")
     pr = sub.add_parser("product")
     pr.add_argument("--rows", type=int, default=8)
     pr.add_argument("--out", type=int, default=8192)

@@ -68,8 +68,12 @@ class GqaAttention:
             return None
         return ("attention", self.n_heads, self.n_kv_heads, self.head_dim)
 
-    def plan_rows(self, seq_rows, add):
-        return self.ops.plan_attention(self.n_heads, self.n_kv_heads, self.head_dim, seq_rows, add)
+    def plan_mode(self, seq_rows):
+        mode = getattr(self.ops, "plan_attention_mode", None)
+        return mode(seq_rows) if mode is not None else None
+
+    def plan_rows(self, seq_rows, add, mode=None):
+        return self.ops.plan_attention(self.n_heads, self.n_kv_heads, self.head_dim, seq_rows, add, mode)
 
     def forward(self, x, ctx, residual=None, norm=None):
         ops, b = self.ops, ctx.batch

@@ -360,9 +360,11 @@ def main() -> int:
         say(f"decode at batch {a.batch} without the prediction heads")
         pts[f"decode_b{a.batch}_trunk_only"] = round(decode_rate(a.batch, a.steps, a.warmup, trunk)[0], 1)
     # the same decode at the headline batch through the scheduler: admission, planning, sampling with the reference's
-    # options (server.py:515-516), finishing
-    say(f"decode at batch {a.batch} through the scheduler")
-    pts[f"decode_b{a.batch}_scheduler"] = round(scheduler_decode_rate(engine, a, cfg, gen), 1)
+    # options (server.py:515-516), finishing. Not at the 7B size: the one run of it there ended with the GPU faulted
+    # and no output, and what caused that is not known.
+    if a.size != "7B":
+        say(f"decode at batch {a.batch} through the scheduler")
+        pts[f"decode_b{a.batch}_scheduler"] = round(scheduler_decode_rate(engine, a, cfg, gen), 1)
     line = {
         "metric": f"decode tok/s at batch {a.batch} ({a.size}, {dkey}); prefill tok/s at {a.prefill_tokens:,} tokens",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,

@@ -54,6 +54,12 @@ CASES = {
     "prompt 512 beside 8 decoding": [(4000 + i, 1) for i in range(8)] + [(1000, 512)],
     "4 prompts of 512": [(0, 512)] * 4,
     "prompt 31 behind 100": [(100, 31)],
+    # steps of a scheduler that feeds prompts of 4,006 tokens under a budget of 2,056 beside decoded tokens
+    "portion 2056": [(0, 2056)],
+    "rest 1950 and next 106": [(2056, 1950), (0, 106)],
+    "1 decoding, portion 2055": [(4006, 1), (106, 2055)],
+    "2 decoding, rest 1845, next 209": [(4008, 1), (4006, 1), (2161, 1845), (0, 209)],
+    "7 decoding, rest 700": [(4020 - i, 1) for i in range(7)] + [(3306, 700)],
 }
 
 

@@ -142,3 +142,45 @@ def test_generation_with_as_many_slots_as_requests(name, max_batch, plan, pool):
     assert got == want
     s.engine.cache.check()
     assert s.engine.free_pages() == s.engine.total_pages()
+
+
+@pytest.mark.parametrize("name", ["E", "D"])
+def test_decoding_requests_of_very_different_lengths_from_captured_graphs(name):
+    """Requests of 30 to 2,000 tokens decode side by side: their key splits are planned request by request on the host
+    (the longest would otherwise run on alone), the plan is made again for every replay of the captured step, and a
+    request that leaves changes the batch's shape. Logits equal the plain model's at every decoded position; the same
+    trace without graphs gives the same plan and, within rounding, the same logits."""
+    from tiny_inference_server_amd.ops import hip_ops
+    folder = H.model_folder(name, "bfloat16")
+    cfg = H.TINY[name]["cfg"]
+    lengths = [2000, 30, 420, 64, 1100, 47] if cfg.max_context >= 2304 else [600, 30, 120, 64, 350, 47]
+    tail = [24, 10, 24, 24, 16, 24]                       # tokens decoded one by one at the end of each request
+    reqs = {f"u{i}": H.random_ids(cfg.vocab_size, n, 130 + i) for i, n in enumerate(lengths)}
+    peak = sum(-(-n // 16) * 16 for n in lengths)
+    got = {}
+    for graphs in (True, False):
+        eng = Engine(folder, dtype="bfloat16", page_size=16, max_tokens=peak, max_requests=len(reqs), use_graphs=graphs)
+        main = {}
+        for (rid, ids), t in zip(reqs.items(), tail):
+            for p in range(0, len(ids) - t, 512):
+                eng.step([(rid, ids[p:min(p + 512, len(ids) - t)], [])])
+        fed = {rid: len(ids) - t for (rid, ids), t in zip(reqs.items(), tail)}
+        planned = 0
+        while any(fed[r] < len(reqs[r]) for r in reqs):
+            live = [r for r in reqs if fed[r] < len(reqs[r])]
+            rows = [(k, fed[r], 1) for k, r in enumerate(live)]
+            planned += hip_ops.uneven_lengths(rows) and len(live) * cfg.n_kv_heads <= hip_ops._ATTN_PLANNED_MAX_WAVES
+            out = eng.step([(r, [reqs[r][fed[r]]], [0]) for r in live])
+            lg = out.logits.float().cpu().clone()
+            for k, r in enumerate(live):
+                main[(r, fed[r])] = lg[k]
+                fed[r] += 1
+        assert planned >= 20                               # most of these steps take the planned lists
+        if graphs:
+            assert eng.graph_replays >= 15 and any(k[0] != "step" and k[2] is not None for k in eng._graphs)
+        got[graphs] = main
+        tol = 2e-2 * max(1.0, max(H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values()))
+        H.compare_with_plain(folder, reqs, main, {}, tol, 0)
+        assert set(main) == {(r, p) for (r, ids), t in zip(reqs.items(), tail) for p in range(len(ids) - t, len(ids))}
+    for key in got[True]:
+        assert (got[True][key] - got[False][key]).abs().max().item() <= 2 * tol, key

@@ -121,3 +121,58 @@ def test_generation_with_as_many_slots_as_requests(name, max_batch, plan, pool):
     assert got == want
     eng.cache.check()
     assert eng.free_pages() == eng.total_pages()
+
+
+class PlanningOps(TorchOps):
+    """The stand-in with the attention mixer's host planning switched on, as the real operations have it: the plan's
+    arrays travel with the step, the stand-in's attention ignores them."""
+
+    def plan_attention_mode(self, seq_rows):
+        from tiny_inference_server_amd.ops.hip_ops import uneven_lengths
+        return "uneven" if uneven_lengths(seq_rows) else None
+
+    def plan_attention(self, n_heads, n_kv_heads, head_dim, seq_rows, add, mode=None):
+        from tiny_inference_server_amd.ops.hip_ops import decode_items
+        if mode != "uneven":
+            return {}
+        entries, most = decode_items(seq_rows, n_heads, n_kv_heads, head_dim)
+        return {("attention_decode_items", n_heads, n_kv_heads): (add(entries), len(entries), most)}
+
+
+def test_parts_plan_again_for_every_replay_of_a_captured_step():
+    """A captured step of requests that differ widely in length carries a work list planned on the host. When the
+    same requests come again the list is planned again, for the new positions, into its place in the step's buffer:
+    after every step the buffer holds, integer for integer, what a fresh plan of that step holds."""
+    from tiny_inference_server_amd.engine.batch import Entry, first_stage_rows, plan_step_batch
+    name = "D"
+    folder = H.model_folder(name, "float32")
+    cfg = H.TINY[name]["cfg"]
+    lengths = [500, 30, 90, 41]
+    reqs = {f"p{i}": H.random_ids(cfg.vocab_size, n, 140 + i) for i, n in enumerate(lengths)}
+    eng = Engine(folder, dtype="float32", page_size=16, max_tokens=1024, max_requests=4, ops=PlanningOps(graphs=True))
+    for rid, ids in reqs.items():
+        eng.step([(rid, ids[:-24], [])])
+    main, checked = {}, 0
+    for t in range(24):
+        entries = [(rid, [ids[len(ids) - 24 + t]], [0]) for rid, ids in reqs.items()]
+        slots = [(eng.requests[rid][0], eng.requests[rid][1]) for rid in reqs]
+        out = eng.step(entries)
+        for k, rid in enumerate(reqs):
+            main[(rid, len(reqs[rid]) - 24 + t)] = out.logits[k].float().clone()
+        graphs = [g for key, g in eng._graphs.items() if key[0] != "step" and key[2] is not None]
+        if not graphs:
+            continue                                        # the shape's first step runs as it is
+        graph = graphs[0]
+        batch_entries = [Entry(s, fed, [e[1][0]], [0]) for (s, fed), e in zip(slots, entries)]
+        mode = eng.model.plan_mode(first_stage_rows(batch_entries))
+        assert mode is not None and mode == graph.mode
+        width = graph.table_at[next(iter(graph.table_at))][1][1]
+        fresh = plan_step_batch(batch_entries, eng.model.lags, eng.model.reads_previous, eng.cache,
+                                eng.spec.max_context, eng.model.plan_rows, table_width=width, mode=mode)
+        assert fresh.layout() == graph.layout
+        want = torch.zeros_like(graph.host)
+        fresh.packer.fill(want)
+        assert torch.equal(graph.host[:fresh.packer.total], want[:fresh.packer.total]), t
+        checked += 1
+    assert checked >= 20 and eng.graph_replays >= 20
+    H.compare_with_plain(folder, reqs, main, {}, TOL["float32"] * scale_of(folder, reqs), 0)

@@ -886,6 +886,8 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
   if (stride > 1 && (!part_o || !part_ml)) return tis_fail("attention_mfma: %d splits need a workspace", stride);
   if (min_steps < -1 || (min_steps == -1 && (!items || n_items < 1 || n_tiles > 0)))
     return tis_fail("attention_mfma: min_steps=%d; -1 goes with a planned list of single rows and no tiles", min_steps);
+  if (min_steps == -1 && ((uintptr_t)items % 16))
+    return tis_fail("attention_mfma: a planned list's entries of four integers must be 16-byte aligned");
   if (min_steps != 0 && n_splits > 1 && !row_splits)
     return tis_fail("attention_mfma: splits chosen item by item (min_steps=%d) need the per-row count array", min_steps);
   if (n_tiles > 0 && tile_max_steps < 1) return tis_fail("attention_mfma: a tile's splits need a longest chain of at least one step");

@@ -35,6 +35,12 @@ struct DeviceState {
 };
 
 constexpr size_t kWorkspaceBytes = 32u << 20;   // what the library may use for split reductions
+// The library's kernels for these shapes split tiles over workgroups and keep partial tiles and arrival flags in the
+// workspace; by tile size times workgroups that can come to 64 MiB, and for such shapes the heuristic reports a need
+// of 0 under the 32 MiB limit. The allocation is therefore longer than the size the library is told, and starts
+// zeroed: both cost nothing, change no choice the library makes, and keep a kernel that overran what it was told,
+// or that met stale flags, inside memory that is the wrapper's own.
+constexpr size_t kWorkspaceAllocated = 160u << 20;
 std::mutex g_mutex;
 std::map<int, DeviceState> g_devices;
 
@@ -44,9 +50,13 @@ int device_state(DeviceState** out) {
   DeviceState& st = g_devices[dev];
   if (!st.handle) {
     if (hipblasLtCreate(&st.handle) != HIPBLAS_STATUS_SUCCESS) return tis_fail("gemm_library: hipblasLtCreate failed");
-    if (hipMalloc(&st.workspace, kWorkspaceBytes) != hipSuccess) {
+    if (hipMalloc(&st.workspace, kWorkspaceAllocated) != hipSuccess) {
       st.handle = nullptr;
-      return tis_fail("gemm_library: no memory for the library's %zu-byte workspace", kWorkspaceBytes);
+      return tis_fail("gemm_library: no memory for the library's %zu-byte workspace", kWorkspaceAllocated);
+    }
+    if (hipMemset(st.workspace, 0, kWorkspaceAllocated) != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
+      st.handle = nullptr;
+      return tis_fail("gemm_library: the workspace could not be cleared");
     }
   }
   *out = &st;

@@ -82,3 +82,25 @@ def test_decode_items_cover_every_step_once_in_waves_of_even_length():
     assert not uneven_lengths([(0, 100, 1), (1, 120, 1), (2, 90, 1)])
     assert uneven_lengths([(0, 100, 1), (1, 4000, 1), (2, 90, 1)])
     assert not uneven_lengths([(0, 100, 2), (2, 4000, 1)]) and not uneven_lengths([(0, 4000, 1)])
+
+
+def test_decoded_tokens_get_a_whole_multiple_of_the_chips_units_in_waves_where_few_more_splits_reach_one():
+    """Equal waves spread evenly over 256 compute units only if their number is a multiple of 256. Where up to twice
+    the splits that the target asks for reach one, that count is taken; where none does, the target's count stays;
+    a context too short for more splits caps it; rows of prompts are not touched."""
+    from tiny_inference_server_amd.ops.hip_ops import attention_launch_plan as plan
+
+    def splits(requests, kv_heads, keys, single=True):
+        return plan(requests, requests, 0, (0, 0), single, keys, kv_heads * 4, kv_heads, 128).n_splits
+    assert splits(64, 3, 4096) == 4          # 768 waves instead of 576
+    assert splits(32, 3, 4096) == 8          # 768 instead of 576
+    assert splits(16, 3, 4096) == 16         # 768 instead of 528
+    assert splits(8, 3, 4096) == 32          # 768 instead of 528
+    assert splits(24, 3, 4096) == 8          # 72 waves a split: no multiple of 256 within 16 splits
+    assert splits(64, 8, 4096) == 1          # 512 waves without any split
+    assert splits(32, 4, 4096) == 4          # 512: the target's count is one already
+    assert splits(64, 3, 300) == 2           # splits of at least 128 keys
+    for requests, kv_heads, keys in ((64, 3, 4096), (16, 3, 4096), (5, 2, 1000), (48, 3, 8192), (7, 1, 70)):
+        s = splits(requests, kv_heads, keys)
+        assert 1 <= s <= max(1, keys // 64) and s < 2 * 512 // (requests * kv_heads) + 2
+    assert splits(64, 3, 4096, single=False) == 11     # 2,048 waves offered to rows of prompts; 12 would be the multiple

@@ -146,15 +146,16 @@ def test_generation_with_as_many_slots_as_requests(name, max_batch, plan, pool):
 
 @pytest.mark.parametrize("name", ["E", "D"])
 def test_decoding_requests_of_very_different_lengths_from_captured_graphs(name):
-    """Requests of 30 to 2,000 tokens decode side by side: their key splits are planned request by request on the host
-    (the longest would otherwise run on alone), the plan is made again for every replay of the captured step, and a
-    request that leaves changes the batch's shape. Logits equal the plain model's at every decoded position; the same
+    """Eighteen requests of 30 to 2,000 tokens decode side by side: their key splits are planned request by request on
+    the host (the longest would otherwise run on alone), the plan is made again for every replay of the captured step,
+    and a request that leaves changes the batch's shape; once fewer than sixteen are left all get the same splits. Logits equal the plain model's at every decoded position; the same
     trace without graphs gives the same plan and, within rounding, the same logits."""
     from tiny_inference_server_amd.ops import hip_ops
     folder = H.model_folder(name, "bfloat16")
     cfg = H.TINY[name]["cfg"]
     lengths = [2000, 30, 420, 64, 1100, 47] if cfg.max_context >= 2304 else [600, 30, 120, 64, 350, 47]
     tail = [24, 10, 24, 24, 16, 24]                       # tokens decoded one by one at the end of each request
+    lengths, tail = lengths + [90 + 11 * i for i in range(12)], tail + [24 - i % 3 for i in range(12)]
     reqs = {f"u{i}": H.random_ids(cfg.vocab_size, n, 130 + i) for i, n in enumerate(lengths)}
     peak = sum(-(-n // 16) * 16 for n in lengths)
     got = {}
@@ -169,7 +170,7 @@ def test_decoding_requests_of_very_different_lengths_from_captured_graphs(name):
         while any(fed[r] < len(reqs[r]) for r in reqs):
             live = [r for r in reqs if fed[r] < len(reqs[r])]
             rows = [(k, fed[r], 1) for k, r in enumerate(live)]
-            planned += hip_ops.uneven_lengths(rows) and len(live) * cfg.n_kv_heads <= hip_ops._ATTN_PLANNED_MAX_WAVES
+            planned += hip_ops.uneven_lengths(rows) and hip_ops.planned_list_pays(len(live), cfg.n_kv_heads)
             out = eng.step([(r, [reqs[r][fed[r]]], [0]) for r in live])
             lg = out.logits.float().cpu().clone()
             for k, r in enumerate(live):

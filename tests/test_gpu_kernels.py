@@ -149,17 +149,22 @@ def dense_reference(q, k, v, group, pos, window=0):
     (6, 3, 48, 16, [16, 17, 300]),
     (12, 3, 128, 16, [4096, 130]),
     # lengths that differ a hundredfold in one step: every request gets splits by its own length
-    (12, 3, 128, 16, [1, 5000, 17, 900, 33, 4096, 64, 2, 8100, 640, 31, 32]),
+    (12, 3, 128, 16, [1, 5000, 17, 900, 33, 4096, 64, 2, 8100, 640, 31, 32, 2500, 7, 129, 1300]),
     (16, 4, 128, 16, [40 + 127 * i for i in range(64)]),
+    (32, 8, 128, 16, [40 + 127 * i for i in range(64)]),      # too many key/value heads for a planned list: same splits for all
     (5, 5, 8, 4, [3, 1100]),
     (4, 1, 256, 32, [65]),
 ])
 def test_paged_attention_single_rows(ops_for, dtype, n_heads, n_kv, hd, page_size, kv_lens):
     """Decode-like rows: the last position of several requests with scattered pages."""
+    from tiny_inference_server_amd.ops import hip_ops
     ops = ops_for(dtype)
     group = n_heads // n_kv
     plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page_size, dtype, seed=20)
     B = len(kv_lens)
+    # which of these cases take the list planned request by request (bfloat16 only) is part of what is tested
+    planned = hip_ops.uneven_lengths([(i, L - 1, 1) for i, L in enumerate(kv_lens)]) and hip_ops.planned_list_pays(B, n_kv)
+    assert planned == (B >= 16 and n_kv < 8)
     q = rnd((B, n_heads * hd), dtype, 21)
     batch = SimpleNamespace(positions=torch.tensor([L - 1 for L in kv_lens], dtype=torch.int32).cuda(),
                             row_seq=torch.arange(B, dtype=torch.int32).cuda(),

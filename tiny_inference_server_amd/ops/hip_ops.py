@@ -105,16 +105,21 @@ def library(name: str) -> _Lib:
 _SKINNY_MAX_ROWS = 32
 _SKINNY_MAX_ROWS_QKV = 64        # the q/k/v projection with norm, rotary and cache write fused stands for three launches
 _ATTN_TARGET_WAVES = 512
+_CHIP_UNITS = 256               # compute units of an MI355X
 _ATTN_PROMPT_TARGET_WAVES = 2048  # what the grid offers where rows of prompts are in the batch ...
 _ATTN_PROMPT_SPLIT_MAX_ROWS = 512 # ... and the batch is small; a long portion fills the chip by its rows alone
 _ATTN_PROMPT_MIN_STEPS = 8         # steps of 32 keys below which a prompt item's split is not worth its merge
 _ATTN_UNEVEN = 1.5              # decoded tokens: from this ratio of the longest request to the mean on, splits are planned
                                 # request by request on the host instead of being the same for all
 _ATTN_DECODE_MAX_SPLITS = 64    # ... and the most that one request may get
-_ATTN_PLANNED_MAX_WAVES = 192   # ... where requests x key/value heads leave room for three splits each: with fewer
-                                # splits to shift between requests the plain grid was as fast or faster (64 uneven
-                                # requests, planned / same splits, us: 3 kv heads 48 / 58, 4: 72 / 70, 8: 162 / 125;
-                                # 16 requests: 18.5 / 20.8, 21.3 / 22.2, 34.3 / 36.7)
+_ATTN_PLANNED_MIN_ROWS = 16     # ... where there are at least this many requests (8: as fast either way) ...
+_ATTN_PLANNED_MAX_WAVES = 384   # ... and requests x key/value heads are at most this: beyond, there are too few splits
+                                # to shift between requests and the plain grid is as fast or faster. A planned list
+                                # aims at one entry (a wave per key/value head) per compute unit, and at
+                                # _ATTN_TARGET_WAVES waves at least. Uneven requests of 128 to 4,200 keys, planned /
+                                # same splits for all, us: 3 kv heads, 96 requests 72 / 87, 64: 43 / 47, 24: 20.5 /
+                                # 24.6; 4 heads, 96: 100 / 103, 48: 39 / 43; 8 heads, 64: 126 / 124, 32: 53.5 / 60.6;
+                                # 1 head, 64: 19.8 / 21.0; with 8 requests 13.2 / 12.4 (3 heads), 23.6 / 21.8 (8)
 _ATTN_MIN_SPLIT_KEYS = 128      # a split shorter than this costs more in merging than it gains in spreading
 _ATTN_TILE_WAVES = 4            # waves of the workgroup that takes a tile of a long portion
 _ATTN_TILE_GROUPS = 512         # workgroups of the tile kernel that the chip runs side by side
@@ -211,11 +216,20 @@ def uneven_lengths(seq_rows) -> bool:
     return longest * n > _ATTN_UNEVEN * total + 2 * n
 
 
+def planned_list_pays(n_rows: int, n_kv_heads: int) -> bool:
+    """Whether single rows of uneven lengths get a planned list rather than the same splits for all."""
+    return n_rows >= _ATTN_PLANNED_MIN_ROWS and n_rows * n_kv_heads <= _ATTN_PLANNED_MAX_WAVES
+
+
+def planned_target_waves(n_kv_heads: int) -> int:
+    return max(_ATTN_TARGET_WAVES, _CHIP_UNITS * n_kv_heads)
+
+
 def decode_items_capacity(n_rows: int, n_kv_heads: int) -> int:
     """Entries of a planned list for `n_rows` single rows: what the splits can add up to, whatever the lengths."""
     # (a multiple of the eight XCDs: workgroups go to them in turn, so the waves of an entry's key/value heads, which
     # read the same pages, then meet in one L2: 162 against 183 us at 8 key/value heads)
-    return -(-(_ATTN_TARGET_WAVES // n_kv_heads + n_rows + 1) // 8) * 8
+    return -(-(planned_target_waves(n_kv_heads) // n_kv_heads + n_rows + 1) // 8) * 8
 
 
 def decode_items_most_splits(n_rows: int, n_heads: int, head_dim: int, workspace_floats=None) -> int:
@@ -234,7 +248,7 @@ def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspa
     pos = np.fromiter((p0 for _, p0, _ in seq_rows), dtype=np.int64, count=n)
     steps = (pos + 32) // 32                                     # a row at position p sees p + 1 keys
     fewest = max(1, _ATTN_MIN_SPLIT_KEYS // 32)
-    even = max(fewest, -(-int(steps.sum()) * n_kv_heads // _ATTN_TARGET_WAVES))
+    even = max(fewest, -(-int(steps.sum()) * n_kv_heads // planned_target_waves(n_kv_heads)))
     most = decode_items_most_splits(n, n_heads, head_dim, workspace_floats)
     splits = np.clip((steps + even // 2) // even, 1, np.minimum(steps, most))
     cap = decode_items_capacity(n, n_kv_heads)
@@ -287,6 +301,15 @@ def attention_launch_plan(n, n_items, n_tiles, tile_steps, single, max_kv_len, n
         # a lone request or two: shorter splits still pay, because so few waves would leave most of the chip idle
         min_keys = _ATTN_MIN_SPLIT_KEYS // 2 if n_items * n_kv_heads <= 8 else _ATTN_MIN_SPLIT_KEYS
         n_splits = max(1, min(-(-target // (n_items * n_kv_heads)), max_kv_len // min_keys))
+        if single and n_splits > 1:
+            # equal waves spread evenly only if their number is a whole multiple of the chip's compute units: a few
+            # more splits that reach one beat the target's count (64 requests over 3 heads at 4,096 keys: 4 splits
+            # 79 us, 3 splits 82; 32 requests: 8 splits 37, 6 splits 40; at 8,192 keys 146 against 163)
+            waves = n_items * n_kv_heads
+            for s in range(n_splits, min(2 * n_splits, max_kv_len // min_keys) + 1):
+                if waves * s % _CHIP_UNITS == 0:
+                    n_splits = s
+                    break
         min_steps = 0 if single else _ATTN_PROMPT_MIN_STEPS
     if n_tiles:
         # a tile's keys are cut so that no workgroup walks a chain of steps much longer than an even share of
@@ -362,7 +385,7 @@ class HipOps:
         plans = {}
         if self.dtype == torch.bfloat16:
             group, cols = n_heads // n_kv_heads, tile_columns(head_dim)
-            if (mode == "uneven" and group <= 64 and len(seq_rows) * n_kv_heads <= _ATTN_PLANNED_MAX_WAVES
+            if (mode == "uneven" and group <= 64 and planned_list_pays(len(seq_rows), n_kv_heads)
                     and all(n == 1 for _, _, n in seq_rows)):
                 entries, most = decode_items(seq_rows, n_heads, n_kv_heads, head_dim)
                 return {("attention_decode_items", group, cols, n_kv_heads): (add(entries), len(entries), most)}
@@ -700,7 +723,7 @@ class HipOps:
             plan = batch.extras.get(("attention_items", group, cols, n_kv_heads))
             if planned is None and plan is None:
                 # a caller that did not plan (a kernel test): plan now, tiles wherever they fit
-                if uneven_lengths(batch.seq_rows) and n * n_kv_heads <= _ATTN_PLANNED_MAX_WAVES:
+                if uneven_lengths(batch.seq_rows) and planned_list_pays(n, n_kv_heads):
                     entries, most = decode_items(batch.seq_rows, n_heads, n_kv_heads, head_dim)
                     planned = (torch.from_numpy(entries).reshape(-1).to(self.device), len(entries), most)
                 else:

@@ -52,7 +52,7 @@ def parse_segments(text: str):
 
 
 def attention_case(ops, a):
-    from .hip_ops import _ATTN_PLANNED_MAX_WAVES, attention_items, decode_items, tile_columns, uneven_lengths
+    from .hip_ops import attention_items, decode_items, planned_list_pays, tile_columns, uneven_lengths
     nh, kvh, hd, ps = a.heads, a.kv_heads, a.head_dim, a.page_size
     segs = parse_segments(a.segments)
     pages = [-(-(p0 + n) // ps) for p0, n in segs]
@@ -73,7 +73,7 @@ def attention_case(ops, a):
                             extras={}, n_rows=rows, max_seq_rows=max(n for _, n in segs), seq_rows=seq_rows)
     # --no-tiles: what the one-wave kernel alone makes of the same rows; --tiles: tiles however little work there is
     import numpy as np
-    if ((uneven_lengths(seq_rows) and len(seq_rows) * kvh <= _ATTN_PLANNED_MAX_WAVES) or a.planned) and not a.same_splits:
+    if ((uneven_lengths(seq_rows) and planned_list_pays(len(seq_rows), kvh)) or a.planned) and not a.same_splits:
         # decoded tokens of requests that differ widely in length: splits planned request by request, as the engine does
         entries, most = decode_items(seq_rows, nh, kvh, hd)
         batch.extras[("attention_decode_items", nh // kvh, tile_columns(hd), kvh)] = (

@@ -278,6 +278,9 @@ def main() -> int:
         # progress on stderr, flushed: names the phase a run was in if it ends without its line
         print(f"[bench] {what}", file=sys.stderr, flush=True)
 
+    # the library's product kernels differ from shape to shape: each new shape is named on stderr before its first launch
+    os.environ.setdefault("TIS_TRACE_SHAPES", "1")
+
     cfg_full = size_config(a.size)
     cfg = cfg_full
     if a.layers and a.layers != cfg_full.n_layers:

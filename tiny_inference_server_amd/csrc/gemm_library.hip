@@ -11,6 +11,8 @@
 // as stored ([N, K] row-major = K x N column-major) under a transpose flag.
 #include <hipblaslt/hipblaslt.h>
 
+#include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -111,6 +113,14 @@ TIS_EXPORT int tis_gemm_library(const void* X, long x_ld, const void* W, const v
       return tis_fail("gemm_library: the library has no algorithm for M=%d N=%d K=%d (status %d)", M, N, K, (int)hs);
     p.algo = found[0].algo;
     it = st->plans.emplace(key, p).first;
+    // TIS_TRACE_SHAPES=1: a line on standard error before the first launch of every new shape, flushed, so that a
+    // run that ends badly has named the last kernel of the library's that was new to it
+    static const bool trace = [] { const char* e = getenv("TIS_TRACE_SHAPES"); return e && e[0] == '1'; }();
+    if (trace) {
+      fprintf(stderr, "[tis-amd] library product, new shape: rows %d, out %d, in %d, residual %d, 32-bit out %d; workspace asked %zu\n",
+              M, N, K, R ? 1 : 0, out_f32 ? 1 : 0, found[0].workspaceSize);
+      fflush(stderr);
+    }
   }
   const Plan& p = it->second;
   const float alpha = 1.f, beta = R ? 1.f : 0.f;

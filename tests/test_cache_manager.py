@@ -115,6 +115,8 @@ def test_random_orders_keep_every_page_accounted_for(seed):
         for name, g in m.groups.items():
             held = sum(g.held(s) for s in live)
             assert held + g.pool.n_free == g.pool.n_pages
+            for s in live:                            # the array form of a table follows every change of the table
+                assert g.line(s).tolist() == g.tables[s]
     for s in list(live):
         m.close_request(s)
     assert m.free_pages() == m.total_pages() and m.n_live == 0

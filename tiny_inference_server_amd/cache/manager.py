@@ -19,6 +19,7 @@ from collections import deque
 from dataclasses import dataclass, field
 from typing import Dict, List, Mapping, Optional, Tuple
 
+import numpy as np
 import torch
 
 from ..parts.spec import PagedKvNeed, StateNeed
@@ -91,6 +92,7 @@ class PageGroup:
         self.plane_of = {k: i for i, k in enumerate(spec.keys)}
         self.tables: Dict[int, List[int]] = {}           # slot -> page id per page index, -1 once released
         self.released: Dict[int, int] = {}               # slot -> number of leading pages already given back
+        self._lines: Dict[int, np.ndarray] = {}          # slot -> its table as an array, until the table changes
         self.storage = None
         if allocate:
             # [plane][page][key or value][kv head][slot in page][head size]; within a page and head the values
@@ -105,6 +107,14 @@ class PageGroup:
     def held(self, slot: int) -> int:
         return sum(1 for p in self.tables.get(slot, ()) if p >= 0)
 
+    def line(self, slot: int) -> np.ndarray:
+        """The slot's table as an int64 array (read only: the same array comes back until the table changes)."""
+        table = self.tables[slot]
+        a = self._lines.get(slot)
+        if a is None or len(a) != len(table):
+            a = self._lines[slot] = np.asarray(table, dtype=np.int64)
+        return a
+
     def pages_for(self, slot: int, n_positions: int) -> int:
         """Pages to take so that positions [0, n_positions) of `slot` are covered."""
         have = len(self.tables.get(slot, ()))
@@ -117,6 +127,8 @@ class PageGroup:
             raise OutOfPages(f"group {self.spec.name!r}: request needs {need} more pages, {self.pool.n_free} are free")
         for _ in range(need):
             table.append(self.pool.take())
+        if need:
+            self._lines.pop(slot, None)
 
     def release_behind(self, slot: int, first_needed: int) -> int:
         """Window groups: give back the pages that lie wholly before the position `first_needed`."""
@@ -128,6 +140,8 @@ class PageGroup:
         for i in range(done, upto):
             self.pool.give_back(table[i])
             table[i] = -1
+        if upto > done:
+            self._lines.pop(slot, None)
         self.released[slot] = max(done, upto)
         return max(0, upto - done)
 
@@ -136,6 +150,7 @@ class PageGroup:
             if p >= 0:
                 self.pool.give_back(p)
         self.released.pop(slot, None)
+        self._lines.pop(slot, None)
 
 
 class CacheManager:
@@ -242,7 +257,7 @@ class CacheManager:
         return self.groups[group].tables[slot]
 
     def check(self) -> None:
-        """Invariants: no page lost, held twice or free twice; no slot both live and free."""
+        """Invariants: no page lost, held twice or free twice; no slot both live and free; no stale copy of a table."""
         for g in self.groups.values():
             g.pool.check()
             seen = set()
@@ -257,5 +272,8 @@ class CacheManager:
                     seen.add(p)
             if len(seen) + g.pool.n_free != g.pool.n_pages:
                 raise CacheError(f"group {g.spec.name!r}: {len(seen)} held + {g.pool.n_free} free != {g.pool.n_pages}")
+            for slot, a in g._lines.items():
+                if slot not in g.tables or a.tolist() != g.tables[slot]:
+                    raise CacheError(f"group {g.spec.name!r}: the kept array of slot {slot}'s table is stale")
         if set(self._free_slots) & set(self._live) or len(self._free_slots) + len(self._live) != self.max_requests:
             raise CacheError("request slots are inconsistent")

@@ -144,91 +144,85 @@ def plan_step_batch(entries: Sequence[Entry], lags: Sequence[int], has_source: S
     page_size = cache.page_size
 
     # block tables: one line per entry, padded; shared by all stages
-    bt_ids = {}
+    bt_ids, tables = {}, {}
     for gname, g in cache.groups.items():
-        width = max(1, max(len(g.tables[e.slot]) for e in entries))
+        lines = [g.line(e.slot) for e in entries]
+        width = max(1, max(len(t) for t in lines))
         if table_width is not None:
             if width > table_width:
                 raise ValueError(f"block tables of {width} pages do not fit the fixed width {table_width}")
             width = table_width
         tab = np.zeros((n_seqs, width), dtype=np.int32)
-        for k, e in enumerate(entries):
-            t = g.tables[e.slot]
-            tab[k, :len(t)] = [p if p >= 0 else 0 for p in t]
+        for k, t in enumerate(lines):
+            np.maximum(t, 0, out=tab[k, :len(t)], casting="unsafe")     # (-1: a page given back)
+        tables[gname] = tab
         bt_ids[gname] = pk.add(tab, tab.shape)
     slots_id = pk.add([e.slot for e in entries])
 
+    # everything below works on arrays over all entries at once: a step may hold hundreds of them
+    starts = np.fromiter((e.start for e in entries), dtype=np.int64, count=n_seqs)
+    n_toks = np.fromiter((len(e.tokens) for e in entries), dtype=np.int64, count=n_seqs)
+    slots = np.fromiter((e.slot for e in entries), dtype=np.int64, count=n_seqs)
+    ends = starts + n_toks
+    if n_seqs and int(ends.max()) > max_context:
+        k = int(np.argmax(ends))
+        raise ValueError(f"request in slot {entries[k].slot} would reach position {int(ends[k]) - 1}, "
+                         f"beyond the model's context of {max_context}")
+    all_tokens = (np.concatenate([np.asarray(e.tokens, dtype=np.int64).reshape(-1) for e in entries])
+                  if n_seqs else np.zeros(0, dtype=np.int64))
+    tok_first = np.cumsum(n_toks) - n_toks                       # where an entry's tokens start in all_tokens
+    for k, e in enumerate(entries):
+        for i in e.want:
+            if not (0 <= i < len(e.tokens)):
+                raise ValueError(f"want index {i} is outside the entry's {len(e.tokens)} tokens")
+    want_entry = np.fromiter((k for k, e in enumerate(entries) for _ in e.want), dtype=np.int64)
+    want_at = np.fromiter((i for e in entries for i in e.want), dtype=np.int64)
+    seq_index = np.arange(n_seqs)
+
     plans = []
-    prev_rows: Optional[List[Tuple[int, int, int]]] = None
-    entry_tokens = [np.asarray(e.tokens, dtype=np.int64).reshape(-1) for e in entries]
-    empty = np.zeros(0, dtype=np.int64)
-
-    def joined(parts):
-        return np.concatenate(parts) if parts else empty
-
+    prev = None                 # the previous stage's (first rows, first positions, row counts)
     for j, lag in enumerate(lags):
-        tokens, positions, row_seq, cu = [], [], [], [0]
-        seq_rows = []
-        source, keep_src, keep_slot = [], [], []
-        n_rows = 0
-        for k, e in enumerate(entries):
-            s, n_tok = e.start, len(e.tokens)
-            end = s + n_tok
-            p0 = max(0, s - lag)
-            n = max(0, end - lag - p0)
-            first_row = n_rows
-            if end > max_context:
-                raise ValueError(f"request in slot {e.slot} would reach position {end - 1}, "
-                                 f"beyond the model's context of {max_context}")
-            pos = np.arange(p0, p0 + n, dtype=np.int64)
-            tokens.append(entry_tokens[k][n_tok - n:])
-            positions.append(pos)
-            row_seq.append(np.full(n, k, dtype=np.int64))
-            n_rows += n
-            cu.append(n_rows)
-            seq_rows.append((first_row, p0, n))
-            if has_source[j]:
-                pfirst, pp0, pn = prev_rows[k]
-                # a row reads the previous stage's row at its position, or the request's kept row before the portion
-                source.append(np.where(pos >= pp0, pfirst + (pos - pp0), -(e.slot + 1)))
-                if pn > 0:
-                    keep_src.append(pfirst + pn - 1)
-                    keep_slot.append(e.slot)
-        tokens, positions, row_seq, source = joined(tokens), joined(positions), joined(row_seq), joined(source)
+        p0 = np.maximum(0, starts - lag)
+        n = np.maximum(0, ends - lag - p0)
+        first = np.cumsum(n) - n
+        n_rows = int(n.sum())
+        row_seq = np.repeat(seq_index, n)
+        positions = np.arange(n_rows) - np.repeat(first - p0, n)
+        # a stage that lags takes the last n of an entry's tokens
+        tokens = all_tokens[np.repeat(tok_first + n_toks - n - p0, n) + positions]
+        seq_rows = list(zip(first.tolist(), p0.tolist(), n.tolist()))
+        source = keep_src = keep_slot = None
+        if has_source[j]:
+            pfirst, pp0, pn = prev
+            # a row reads the previous stage's row at its position, or the request's kept row before the portion
+            source = np.where(positions >= np.repeat(pp0, n), np.repeat(pfirst - pp0, n) + positions,
+                              np.repeat(-(slots + 1), n))
+            kept = pn > 0
+            keep_src, keep_slot = (pfirst + pn - 1)[kept], slots[kept]
         ws = {}
-        for gname, g in cache.groups.items():
-            arr = np.empty(n_rows, dtype=np.int32)
-            for k, e in enumerate(entries):
-                first_row, p0, n = seq_rows[k]
-                if n:
-                    p = np.arange(p0, p0 + n)
-                    arr[first_row:first_row + n] = np.asarray(g.tables[e.slot], dtype=np.int64)[p // page_size] \
-                        * page_size + p % page_size
-            ws[gname] = pk.add(arr)
-        want, valid = [], []
-        for k, e in enumerate(entries):
-            first_row, p0, n = seq_rows[k]
-            for i in e.want:
-                if not (0 <= i < len(e.tokens)):
-                    raise ValueError(f"want index {i} is outside the entry's {len(e.tokens)} tokens")
-                p = e.start + i - lag
-                ok = p >= p0 and n > 0
-                want.append(first_row + (p - p0) if ok else -1)
-                valid.append(ok)
+        for gname in cache.groups:
+            # (a new position never lies in a page that was given back, so the padded table serves)
+            t = tables[gname]
+            ws[gname] = pk.add(t[row_seq, positions // page_size].astype(np.int64) * page_size + positions % page_size)
+        wp = starts[want_entry] + want_at - lag
+        ok = (wp >= p0[want_entry]) & (n[want_entry] > 0)
+        want = np.where(ok, first[want_entry] + wp - p0[want_entry], -1)
         extra = {}
         if plan_rows is not None:
             extra = plan_rows(seq_rows, pk.add, mode) if mode is not None else plan_rows(seq_rows, pk.add)
+        live = n > 0
         plans.append(dict(
             extra=extra, lag=lag, n_rows=n_rows, tokens=pk.add(tokens), positions=pk.add(positions),
-            row_seq=pk.add(row_seq), cu=pk.add(cu), ws=ws,
+            row_seq=pk.add(row_seq), cu=pk.add(np.concatenate(([0], np.cumsum(n)))), ws=ws,
             source=pk.add(source) if has_source[j] else None,
             keep_src=pk.add(keep_src) if has_source[j] else None,
             keep_slot=pk.add(keep_slot) if has_source[j] else None,
-            keep_count=len(keep_src), previous_rows=int((source >= 0).sum()) if has_source[j] else 0,
-            want=pk.add(want), valid=valid, seq_rows=seq_rows,
-            max_kv=max([p0 + n for _, p0, n in seq_rows if n > 0] or [0]),
-            max_rows=max([n for _, _, n in seq_rows] or [0])))
-        prev_rows = seq_rows
+            keep_count=int(len(keep_src)) if has_source[j] else 0,
+            previous_rows=int((source >= 0).sum()) if has_source[j] else 0,
+            want=pk.add(want), valid=ok.tolist(), seq_rows=seq_rows,
+            max_kv=int((p0 + n)[live].max()) if live.any() else 0,
+            max_rows=int(n.max()) if n_seqs else 0))
+        prev = (first, p0, n)
 
     return StepPlan(list(entries), pk, bt_ids, slots_id, plans)
 

@@ -174,14 +174,12 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
     def cut(segments, per_item):
         if not segments:
             return none, (0, 0)
-        firsts, counts, keys = [], [], []
-        for first, p0, n in segments:
-            r = np.arange(0, n, per_item, dtype=np.int64)
-            cnt = np.minimum(per_item, n - r)
-            firsts.append(first + r)
-            counts.append(cnt)
-            keys.append(p0 + r + cnt)
-        firsts, counts, keys = np.concatenate(firsts), np.concatenate(counts), np.concatenate(keys)
+        first, p0, n = np.asarray(segments, dtype=np.int64).reshape(-1, 3).T
+        k = -(-n // per_item)                                          # items of each segment
+        r = (np.arange(int(k.sum())) - np.repeat(np.cumsum(k) - k, k)) * per_item    # an item's first row in its segment
+        counts = np.minimum(per_item, np.repeat(n, k) - r)
+        firsts = np.repeat(first, k) + r
+        keys = np.repeat(p0, k) + r + counts
         # those with the most keys first: under a causal mask the last rows of a prompt are the longest, and
         # started last they would run on alone while the rest of the chip idles
         order = np.argsort(-keys, kind="stable")

@@ -105,6 +105,49 @@ def test_repeated_prompt_steps_are_replayed(name):
     assert eng.free_pages() == eng.total_pages()
 
 
+def test_tiles_beside_items_on_two_streams_eager_and_replayed():
+    """A step of one long portion (tiles of a workgroup, on the library's second stream) beside a shorter one and three
+    decoded tokens (items, one wave each, on the first): the two kernels run side by side and meet again before the
+    merge. The same shape comes four times with other tokens; the first runs kernel by kernel, the last from a captured
+    graph whose branches fork and join. Logits at the ends of both portions and of the decoded tokens equal the plain
+    model's every time they are checked."""
+    from tiny_inference_server_amd.ops import hip_ops
+    name = "E"                                            # the headline model's layer sizes: 12 heads of 128 over 3
+    folder = H.model_folder(name, "bfloat16")
+    cfg = H.TINY[name]["cfg"]
+    eng = Engine(folder, dtype="bfloat16", page_size=16, max_tokens=4096, max_requests=8)
+    long, short, deep = 1700, 300, 70
+    seen = []
+    plan_attention = eng.ops.plan_attention
+
+    def spy(*a, **k):
+        out = plan_attention(*a, **k)
+        seen.extend((v[1], v[3]) for key, v in out.items() if key[0] == "attention_items")
+        return out
+    eng.ops.plan_attention = spy
+    for rep in range(4):
+        reqs = {f"t{rep}_{i}": H.random_ids(cfg.vocab_size, n, 500 + 10 * rep + i) for i, n in enumerate([long, short, deep, deep + 3, deep + 9])}
+        names = list(reqs)
+        for rid in names[2:]:                             # three requests already deep enough to decode
+            eng.step([(rid, reqs[rid][:-1], [])])
+        seen.clear()
+        out = eng.step([(names[0], reqs[names[0]], [long - 1]), (names[1], reqs[names[1]], [0, short - 1])] +
+                       [(rid, reqs[rid][-1:], [0]) for rid in names[2:]])
+        assert any(items > 0 and tiles > 0 for items, tiles in seen)          # both kernels had work in this step
+        lg = out.logits.float().cpu().clone()
+        torch.cuda.synchronize()
+        if rep in (0, 3):
+            main = {(names[0], long - 1): lg[0], (names[1], 0): lg[1], (names[1], short - 1): lg[2]}
+            main.update({(rid, len(reqs[rid]) - 1): lg[3 + k] for k, rid in enumerate(names[2:])})
+            scale = max(1.0, max(H.plain_logits(folder, ids)[0].abs().max().item() for ids in reqs.values()))
+            H.compare_with_plain(folder, reqs, main, {}, 2e-2 * scale, 0)
+        for rid in names:
+            eng.close(rid)
+    assert eng.graph_replays >= 1 and hip_ops._side_streams
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()
+
+
 @pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("D", "bfloat16"), ("C", "bfloat16")])
 def test_requests_follow_each_other_through_one_slot(name, dtype):
     """As many slots as live requests: one. Every request takes over its predecessor's slot at the same place in the

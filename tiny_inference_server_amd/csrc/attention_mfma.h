@@ -18,6 +18,12 @@ int tis_attention_mfma(const void* q, long q_ld, const void* plane, const int* b
                        int n_heads, int n_kv_heads, int head_dim, int page_size, int window, float scale, int n_splits,
                        int min_steps, int tile_splits, int tile_max_steps, int* row_splits, hipStream_t stream);
 
+// A second stream (default priority, as `stream` must have) on which a call that holds both tiles and items runs its
+// tile kernel, beside the items' kernel on `stream`; the two meet again before the merge, and everything after the
+// call on `stream` waits for both. Per device; null (the start) keeps everything on `stream`. The stream must outlive
+// every later call on that device. Works under stream capture (the graph gets two branches).
+int tis_attention_mfma_side_stream(hipStream_t side);
+
 // The same attention for callers that cannot allocate device memory and have no workspace to bring: code under HIP
 // graph capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference, whose
 // attention kernels get their partial-result buffers from the tensor framework (paged_attention_kernels.py:229-231).

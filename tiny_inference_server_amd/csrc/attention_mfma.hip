@@ -857,6 +857,29 @@ TIS_EXPORT int tis_attention_mfma_tile_columns() { return 16 * TNB; }
 // min_steps == -1: `items` holds n_items entries of four integers, one per wave and key/value head, planned on the
 // host for single rows: (row, split + 65536 * splits of the row, position, block-table line), row < 0 for padding;
 // n_splits is then the most splits any row may have (the partial results' stride).
+// A second stream for the tile kernel where a step has tiles and items: the two kernels share no rows, one is bound
+// by the matrix cores and LDS, the other by memory, and side by side they take less than one after the other. Set
+// once per device by the owner of the streams (null: everything on the caller's stream). Both streams must have
+// the default priority.
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+};
+static SideStream g_side[64];
+
+TIS_EXPORT int tis_attention_mfma_side_stream(hipStream_t side) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return tis_fail("attention_mfma: no current device");
+  SideStream& st = g_side[dev];
+  if (side && !st.fork) {
+    if (hipEventCreateWithFlags(&st.fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&st.join, hipEventDisableTiming) != hipSuccess)
+      return tis_fail("attention_mfma: no events for the second stream");
+  }
+  st.stream = side;
+  return 0;
+}
+
 static int attention_launch(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
                             const int* row_seq, const int* positions, const int* items, int n_items, int nb,
                             const int* tiles, int n_tiles, void* out, long out_ld, float* part_o,
@@ -898,6 +921,18 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
     return tis_fail("attention_mfma: q, out and the cache plane must be 16-byte aligned with row strides in steps of 8");
   const float scale_log2 = scale * 1.4426950408889634f;
   int rc = 0;
+  hipStream_t tile_stream = stream;
+  const SideStream* side = nullptr;
+  if (n_items > 0 && n_tiles > 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && g_side[dev].stream && g_side[dev].stream != stream) {
+      side = &g_side[dev];
+      // the tiles wait for what came before this call, not for the items
+      if (hipEventRecord(side->fork, stream) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
+        return tis_fail("attention_mfma: the second stream could not be joined to the first");
+      tile_stream = side->stream;
+    }
+  }
   if (n_items > 0) {
     dim3 grid(n_items, n_kv_heads, min_steps < 0 ? 1 : n_splits);
 #define LAUNCH(NBV, PSV)                                                                                              \
@@ -921,7 +956,7 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
   if (n_tiles > 0) {
     dim3 grid(n_tiles, n_kv_heads, tile_splits);
 #define LAUNCH(PSV)                                                                                                   \
-  attention_tile_kernel<PSV><<<grid, TW * 64, 0, stream>>>(                                                      \
+  attention_tile_kernel<PSV><<<grid, TW * 64, 0, tile_stream>>>(                                                      \
       (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)tiles,     \
       (bf16*)out, out_ld, part_o, (float2*)part_ml, group, n_kv_heads, n_heads, page_size, window, scale_log2,   \
       tile_splits, tile_max_steps, stride, row_splits)
@@ -929,6 +964,9 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
     else LAUNCH(false);
 #undef LAUNCH
     rc = tis_launch_status("attention_tile");
+    if (side && (hipEventRecord(side->join, side->stream) != hipSuccess ||
+                 hipStreamWaitEvent(stream, side->join, 0) != hipSuccess))
+      return tis_fail("attention_mfma: the first stream could not wait for the second");
     if (rc) return rc;
   }
   if (stride > 1) {

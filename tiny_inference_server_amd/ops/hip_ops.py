@@ -85,6 +85,7 @@ _SIGNATURES["gemm_library"] = ("tis_gemm_library", {
     "tis_gemm_library": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _I, _P],
 })
 _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
+    "tis_attention_mfma_side_stream": [_P],
     "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F,
                            _I, _I, _I, _I, _P, _P],
 })
@@ -329,6 +330,18 @@ def attention_launch_plan(n, n_items, n_tiles, tile_steps, single, max_kv_len, n
     rs_offset = n * n_heads * stride * (head_dim + 2)
     return AttentionLaunch(n_splits, min_steps, tile_splits, tile_max_steps, stride, ml_offset, rs_offset,
                            rs_offset + n if stride > 1 else 0)
+
+
+_side_streams = {}
+
+
+def _side_stream(device_index: int):
+    """The device's second stream (default priority), on which the attention library runs a step's tiles beside its
+    items. One per device for the life of the process: the library keeps its handle."""
+    s = _side_streams.get(device_index)
+    if s is None:
+        s = _side_streams[device_index] = torch.cuda.Stream(torch.device("cuda", device_index))
+    return s
 
 
 def _rows_view(t: torch.Tensor, what: str):
@@ -749,6 +762,8 @@ class HipOps:
             lib = self._attn_mfma.get(head_dim)
             if lib is None:
                 lib = self._attn_mfma[head_dim] = library(f"attention_mfma@{head_dim}")
+                with torch.cuda.device(self.device):
+                    lib.tis_attention_mfma_side_stream(c_void_p(_side_stream(self._device_index).cuda_stream))
                 built = lib.cdll.tis_attention_mfma_tile_columns()
                 if built != cols:
                     raise KernelError(f"attention: the kernel's tiles hold {built} columns a wave, the planner "

@@ -129,3 +129,28 @@ def test_slots_run_out_with_a_clear_error():
     m.open_request(), m.open_request()
     with pytest.raises(CacheError, match="all 2 request slots"):
         m.open_request()
+
+
+def test_the_spare_request_lives_beside_what_was_asked_for():
+    """A manager with a spare request: its slot, state line and pages come on top of the slots and pages asked for and
+    are counted by nobody; it cannot be closed; everything else behaves as without it."""
+    needs = {"a": PagedKvNeed(2, 8), "b": PagedKvNeed(2, 8, window=6), "s": StateNeed((4,), "float32")}
+    m = CacheManager(needs, 4, 5, 2, torch.float32, "cpu", spare_positions=3)
+    assert m.spare_slot == 2 and m.n_live == 0
+    assert m.free_pages() == m.total_pages() == {"kv2x8": 5, "kv2x8w6": 5}
+    assert m.states["s"].shape == (3, 4) and all(g.storage.shape[1] == 6 for g in m.groups.values())
+    assert [len(g.tables[2]) for g in m.groups.values()] == [1, 1]
+    a, b = m.open_request(), m.open_request()
+    assert {a, b} == {0, 1}
+    with pytest.raises(CacheError, match="all 2 request slots"):
+        m.open_request()
+    m.grow(a, 12), m.grow(b, 8)                       # all five pages of the full group
+    assert m.free_pages()["kv2x8"] == 0 and not m.can_grow({b: 9})
+    spare_pages = {name: list(g.tables[2]) for name, g in m.groups.items()}
+    assert all(p not in g.tables[a] + g.tables[b] for name, g in m.groups.items() for p in spare_pages[name])
+    with pytest.raises(CacheError, match="spare"):
+        m.close_request(2)
+    m.check()
+    m.close_request(a), m.close_request(b)
+    assert m.free_pages() == m.total_pages() and m.n_live == 0
+    m.check()

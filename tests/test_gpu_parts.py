@@ -385,7 +385,7 @@ def test_window_layers_get_pages_of_their_own_and_give_them_back(dtype, tol):
     assert worst <= tol * scale, worst
     eng.close("a")
     eng.cache.check()
-    assert all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups.values())
+    assert eng.cache.free_pages() == eng.cache.total_pages()
     ARCHITECTURES.unregister("WindowedToy")
 
 

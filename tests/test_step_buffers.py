@@ -176,3 +176,45 @@ def test_parts_plan_again_for_every_replay_of_a_captured_step():
         checked += 1
     assert checked >= 20 and eng.graph_replays >= 20
     H.compare_with_plain(folder, reqs, main, {}, TOL["float32"] * scale_of(folder, reqs), 0)
+
+
+def shrinking_batch(reqs, prompt):
+    """All requests decode side by side after their prompts; they are of different lengths, so the batch shrinks one
+    request at a time."""
+    steps = [{"step": i, "entries": [{"id": rid, "tokens": ids[:prompt], "want": []}], "end": []}
+             for i, (rid, ids) in enumerate(reqs.items())]
+    fed = {rid: prompt for rid in reqs}
+    while any(fed[r] < len(reqs[r]) for r in reqs):
+        live = [r for r in reqs if fed[r] < len(reqs[r])]
+        steps.append({"step": len(steps), "entries": [{"id": r, "tokens": [reqs[r][fed[r]]], "want": [0]} for r in live],
+                      "end": [r for r in live if fed[r] + 1 == len(reqs[r])]})
+        for r in live:
+            fed[r] += 1
+    return steps
+
+
+@pytest.mark.parametrize("backend", [pytest.param("hip", marks=pytest.mark.gpu), "torch"])
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("D", "bfloat16")])
+def test_a_batch_that_shrinks_request_by_request_meets_few_shapes(name, dtype, backend):
+    """Thirteen requests decode side by side and end one after the other. Steps of nine and more are filled up to 16
+    lines with the cache manager's own request, so sizes 13 down to 9 share one captured shape (two with the table
+    width growing), sizes 8 down to 1 have their own; the filler's lines never come back, and every request's logits
+    equal the plain model's, also right after a neighbour has left."""
+    vocab = H.TINY[name]["cfg"].vocab_size
+    reqs = {f"k{i}": H.random_ids(vocab, 24 + 3 * i, 700 + i) for i in range(13)}
+    page = H.TINY[name]["page_size"]
+    peak = sum(-(-len(ids) // page) * page for ids in reqs.values())
+    if backend == "torch":
+        folder, eng = engine_for(name, dtype, max_tokens=peak, max_requests=13)
+    else:
+        folder = H.model_folder(name, "float32" if dtype == "float32" else "bfloat16")
+        eng = Engine(folder, dtype=dtype, page_size=page, max_tokens=peak, max_requests=13)
+    assert eng.use_decode_graphs and eng.cache.spare_slot == 13
+    steps = shrinking_batch(reqs, 20)
+    main, _ = H.run_trace(eng, steps, heads=False)
+    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0, steps)
+    sizes = sorted({k[0] for k in eng._graphs if k[0] != "step"} | {k[0] for k in eng._graph_seen if k[0] != "step"})
+    assert sizes == [1, 2, 3, 4, 5, 6, 7, 8, 16]
+    assert eng.graph_replays > 30
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages() and eng.cache.n_live == 0

@@ -161,13 +161,21 @@ class CacheManager:
     """
 
     def __init__(self, needs: Mapping[str, object], page_size: int, n_pages: int, max_requests: int, dtype,
-                 device, allocate: bool = True):
+                 device, allocate: bool = True, spare_positions: int = 0):
+        """spare_positions > 0: beside the `max_requests` slots and `n_pages` pages there is one request of the
+        manager's own, live from the start with that many positions covered (`spare_slot`; its slot, state and pages
+        come on top and are not counted by free_pages, total_pages and n_live): what a step of a fixed shape is
+        filled up with when fewer requests come than the shape has lines."""
         if page_size < 1:
             raise CacheError(f"page size must be at least 1, got {page_size}")
         if max_requests < 1:
             raise CacheError(f"max_requests must be at least 1, got {max_requests}")
         self.page_size = page_size
         self.max_requests = max_requests
+        self.spare_slot: Optional[int] = max_requests if spare_positions > 0 else None
+        self._spare_pages = -(-spare_positions // page_size) if spare_positions > 0 else 0
+        n_slots = max_requests + (1 if spare_positions > 0 else 0)
+        n_pages = n_pages + self._spare_pages
         self.dtype, self.device = dtype, device
         specs: Dict[Tuple[int, int, int], GroupSpec] = {}
         self.group_of: Dict[str, str] = {}
@@ -186,18 +194,23 @@ class CacheManager:
                 self.states[key] = None
                 if allocate:
                     dt = {"compute": dtype, "float32": torch.float32, "int32": torch.int32}[need.dtype]
-                    self.states[key] = torch.zeros((max_requests,) + tuple(need.shape), dtype=dt, device=device)
+                    self.states[key] = torch.zeros((n_slots,) + tuple(need.shape), dtype=dt, device=device)
             elif need is not None:
                 raise CacheError(f"cache key {key!r}: unknown kind of need {need!r}")
         self.groups: Dict[str, PageGroup] = {
             s.name: PageGroup(s, n_pages, page_size, dtype, device, allocate) for s in specs.values()}
         self._free_slots = deque(range(max_requests))
         self._live: Dict[int, bool] = {}
+        if self.spare_slot is not None:
+            self._live[self.spare_slot] = True
+            for g in self.groups.values():
+                g.tables[self.spare_slot] = []
+                g.grow(self.spare_slot, spare_positions)
 
     # ---- requests ------------------------------------------------------------------------------------
     @property
     def n_live(self) -> int:
-        return len(self._live)
+        return len(self._live) - (1 if self.spare_slot is not None else 0)
 
     def open_request(self) -> int:
         if not self._free_slots:
@@ -212,6 +225,8 @@ class CacheManager:
         return slot
 
     def close_request(self, slot: int) -> None:
+        if slot == self.spare_slot:
+            raise CacheError("the spare request stays live as long as the manager")
         if slot not in self._live:
             raise CacheError(f"request slot {slot} is not live (closed twice?)")
         del self._live[slot]
@@ -251,7 +266,7 @@ class CacheManager:
         return {name: g.pool.n_free for name, g in self.groups.items()}
 
     def total_pages(self) -> Dict[str, int]:
-        return {name: g.pool.n_pages for name, g in self.groups.items()}
+        return {name: g.pool.n_pages - self._spare_pages for name, g in self.groups.items()}
 
     def block_table(self, group: str, slot: int) -> List[int]:
         return self.groups[group].tables[slot]
@@ -275,5 +290,5 @@ class CacheManager:
             for slot, a in g._lines.items():
                 if slot not in g.tables or a.tolist() != g.tables[slot]:
                     raise CacheError(f"group {g.spec.name!r}: the kept array of slot {slot}'s table is stale")
-        if set(self._free_slots) & set(self._live) or len(self._free_slots) + len(self._live) != self.max_requests:
+        if set(self._free_slots) & set(self._live) or len(self._free_slots) + self.n_live != self.max_requests:
             raise CacheError("request slots are inconsistent")

@@ -25,6 +25,12 @@ _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.
            torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
 
 
+# Captured steps of single tokens: up to this many requests a step has its own shape, beyond it the next multiple of
+# the step below (the filler lines cost a row of every product and a wave of attention over three keys each)
+_EXACT_DECODE_SHAPES = 8
+_DECODE_SHAPE_STEP = 8
+
+
 def resolve_dtype(dtype):
     try:
         return _DTYPES[dtype]
@@ -70,16 +76,24 @@ class Engine:
                 raise ValueError("give the cache's size as max_tokens or n_pages")
             n_pages = -(-int(max_tokens) // page_size)
         self.page_size = page_size
-        self.cache = CacheManager(self.model.cache_needs(), page_size, n_pages, max_requests, self.dtype, self.device)
+        # decode steps are replayed from captured graphs where the kernels allow it
+        can = bool(use_graphs) and bool(getattr(ops, "supports_graphs", False))
+        self.use_graphs = can and self.model.graph_safe                          # any step whose shape repeats
+        self.use_decode_graphs = can and self.model.graph_safe_single_rows       # steps of single tokens
+        # A captured step of single tokens has a fixed number of lines. Steps of nine requests and more are filled up
+        # to the next multiple of eight with lines of a request of the cache manager's own (a token at a fixed
+        # position, in a slot and a page beyond the ones that were asked for), so that a batch that shrinks request
+        # by request meets a few shapes and not one per size.
+        self.cache = CacheManager(self.model.cache_needs(), page_size, n_pages, max_requests, self.dtype, self.device,
+                                  spare_positions=self.model.max_lag + 1 if self.use_decode_graphs else 0)
+        self.max_requests = max_requests
         self.requests: Dict[Hashable, Tuple[int, int]] = {}      # id -> (slot, positions fed)
         # a slot is handed to request after request; what a captured step keeps about "the requests it holds" must
         # change when a slot changes hands, so every admission gets a number and a slot remembers its occupant's
         self._admissions = 0
         self._slot_admission: Dict[int, int] = {}
-        # decode steps are replayed from captured graphs where the kernels allow it
-        can = bool(use_graphs) and bool(getattr(ops, "supports_graphs", False))
-        self.use_graphs = can and self.model.graph_safe                          # any step whose shape repeats
-        self.use_decode_graphs = can and self.model.graph_safe_single_rows       # steps of single tokens
+        if self.cache.spare_slot is not None:
+            self._slot_admission[self.cache.spare_slot] = 0
         # an operations object without a device to capture on (a test's stand-in) may ask for the same host logic
         # with plain launches in place of replays
         self._capture_graphs = not getattr(ops, "emulates_graphs", False)
@@ -334,6 +348,11 @@ class Engine:
         width = -(-pages // self.graph_table_pages) * self.graph_table_pages
         # (what the parts' planning says about the step, e.g. requests of very different lengths, changes the launches)
         mode = self.model.plan_mode(first_stage_rows(batch_entries))
+        n_real = len(batch_entries)
+        if n_real > _EXACT_DECODE_SHAPES and self.cache.spare_slot is not None:
+            lines = -(-n_real // _DECODE_SHAPE_STEP) * _DECODE_SHAPE_STEP
+            filler = Entry(self.cache.spare_slot, self.model.max_lag, [0], [0])
+            batch_entries = list(batch_entries) + [filler] * (lines - n_real)
         key = (len(batch_entries), width, mode)
         graph = self._graphs.get(key)
         if graph is not None:
@@ -344,7 +363,7 @@ class Engine:
                 if e.start + 1 > self.spec.max_context:
                     raise ValueError(f"request in slot {e.slot} would pass the model's context of {self.spec.max_context}")
             self.graph_replays += 1
-            return graph.run_same_requests(batch_entries)
+            return graph.run_same_requests(batch_entries)[:n_real]
         plan = plan_step_batch(batch_entries, self.model.lags, self.model.reads_previous, self.cache,
                                self.spec.max_context, self.model.plan_rows, table_width=width, mode=mode)
         if graph is None:
@@ -357,9 +376,9 @@ class Engine:
                 for st in step.stages:
                     st.max_kv_len = width * self.page_size
                 outs = self.model.forward(step, self.cache)
-                return self.model.logits(outs[0].hidden, step.stages[0].want_index, len(batch_entries))
+                return self.model.logits(outs[0].hidden, step.stages[0].want_index, len(batch_entries))[:n_real]
             self._make_room(lambda k: k[0] != "step", self.max_decode_graphs)
             graph = self._graphs[key] = DecodeGraph(self, plan, width * self.page_size, occupants,
                                                     capture=self._capture_graphs, mode=mode)
         self.graph_replays += 1
-        return graph.run(plan, occupants)
+        return graph.run(plan, occupants)[:n_real]

@@ -547,7 +547,8 @@ def test_skinny_product_with_fused_norm_residual_and_gate(ops_for, M, N, K):
 def test_projection_with_rotary_and_cache_write(ops_for, dtype, M, n_heads, n_kv, hd, page_size, interleaved):
     """q/k/v projection + rotary + cache write: one kernel for few bfloat16 rows, two otherwise; same results."""
     ops, ref = ops_for(dtype), TorchOps(dtype=dtype)
-    K, n_pages, max_ctx = 96, -(-M // page_size) + 3, 300
+    # (the headline model's width for 33 and 64 rows of its geometry: four row blocks of the few-row kernel at a real size)
+    K, n_pages, max_ctx = (1536 if hd == 128 and M in (33, 64) else 96), -(-M // page_size) + 3, 300
     N = (n_heads + 2 * n_kv) * hd
     j = torch.arange(hd // 2)
     ang = torch.outer(torch.arange(max_ctx).float(), 1.0 / torch.pow(torch.tensor(1e4), (2 * j.float()) / hd))

@@ -7,7 +7,7 @@ package, without editing the code that does the lookup.
 """
 from __future__ import annotations
 
-from typing import Callable, Dict, Generic, Iterator, TypeVar
+from typing import Dict, Generic, Iterator, TypeVar
 
 T = TypeVar("T")
 

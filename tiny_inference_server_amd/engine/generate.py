@@ -1,7 +1,7 @@
 """The Python entry point: token ids in, generated token ids out."""
 from __future__ import annotations
 
-from typing import List, Optional, Sequence
+from typing import Optional, Sequence
 
 from ..sampling.params import SamplingParams
 from .engine import Engine

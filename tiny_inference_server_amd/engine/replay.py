@@ -17,8 +17,6 @@ import os
 import sys
 from typing import IO, Optional
 
-import numpy as np
-
 from .engine import Engine
 
 

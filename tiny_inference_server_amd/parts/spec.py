@@ -15,7 +15,7 @@ and runs the spec and never asks which architecture it came from.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Mapping, Optional, Tuple
+from typing import Any, Mapping, Optional, Tuple
 
 
 @dataclass(frozen=True)

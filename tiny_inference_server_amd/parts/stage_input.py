@@ -1,8 +1,6 @@
 """Stage inputs: where the rows of a stage come from."""
 from __future__ import annotations
 
-import torch
-
 from .base import STAGE_INPUTS, build_part, to_compute
 from .spec import StateNeed
 

@@ -181,6 +181,34 @@ def test_paged_attention_single_rows(ops_for, dtype, n_heads, n_kv, hd, page_siz
         assert not torch.allclose(got[0].view(n_heads, hd).double(), bad, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("window", [1000, 500])
+def test_single_rows_of_uneven_lengths_behind_a_window(ops_for, window):
+    """Decoded tokens of requests that differ widely in length, in a layer that sees a window ending inside a page:
+    the splits are planned from what each row sees (the window's keys), not from its request's length."""
+    from tiny_inference_server_amd.ops import hip_ops
+    ops = ops_for(torch.bfloat16)
+    n_heads, n_kv, hd, page_size = 12, 3, 128, 16
+    kv_lens = [1, 5000, 17, 900, 33, 4096, 64, 2, 8100, 640, 31, 32, 2500, 7, 129, 1300, 151, 999]
+    seq_rows = [(i, L - 1, 1) for i, L in enumerate(kv_lens)]
+    assert hip_ops.uneven_lengths(seq_rows, window) and hip_ops.planned_list_pays(len(kv_lens), n_kv)
+    entries, _ = hip_ops.decode_items(seq_rows, n_heads, n_kv, hd, window=window)
+    live = entries[entries[:, 0] >= 0]
+    for i, L in enumerate(kv_lens):          # no row gets more splits than its window has steps of 32 keys
+        steps = (L + 31 - (max(0, L - window) & ~31)) // 32
+        assert 1 <= (live[live[:, 0] == i][:, 1] >> 16).max() <= steps
+    plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page_size, torch.bfloat16, seed=27)
+    B = len(kv_lens)
+    q = rnd((B, n_heads * hd), torch.bfloat16, 28)
+    batch = SimpleNamespace(positions=torch.tensor([L - 1 for L in kv_lens], dtype=torch.int32).cuda(),
+                            row_seq=torch.arange(B, dtype=torch.int32).cuda(),
+                            block_tables={"g": tables.cuda()}, max_kv_len=max(kv_lens), extras={},
+                            n_rows=B, max_seq_rows=1, seq_rows=seq_rows)
+    got = ops.paged_attention(q.cuda(), plane.cuda(), batch, "g", n_heads, n_kv, hd, window=window).cpu()
+    for i, L in enumerate(kv_lens):
+        want = dense_reference(q[i].view(n_heads, hd), ks[i], vs[i], n_heads // n_kv, L - 1, window)
+        torch.testing.assert_close(got[i].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("page_size", [16, 32])
 def test_single_rows_walking_a_long_context_without_splits(ops_for, monkeypatch, page_size):
     """With no key splits one wave walks a request's whole context alone: thousands of keys, hundreds of steps,
@@ -488,29 +516,58 @@ def test_sampling_reference_vectors(ops_for):
     assert ops.sample(lg.cuda(), *args, one(2.0), one(0.5), one(5, torch.int32), torch.tensor([0, 1], dtype=torch.int32).cuda()).item() == 7
 
 
-@pytest.mark.parametrize("M", [33, 64, 200])
+@pytest.mark.parametrize("M", [33, 64, 65, 200, 777])
 @pytest.mark.parametrize("N,K", [(96, 64), (1000, 96), (2304, 1536)])
 def test_product_with_norm_residual_and_gate_for_many_rows(ops_for, M, N, K):
-    """Above 32 rows the same calls run as separate kernels around the library's product; the results agree with the
-    reference's order of operations (norm rounded to bfloat16, product, gating)."""
+    """More rows than a workgroup of the few-row kernel takes: panels of rows (any width), or, at a width from the
+    library's list, separate kernels around the library's product. The results agree with the reference's order of
+    operations (norm rounded to bfloat16, product, gating)."""
     ops, ref = ops_for(torch.bfloat16), TorchOps(dtype=torch.bfloat16)
     x, w, res = rnd((M, K), torch.bfloat16, 80, 2.0), rnd((N, K), torch.bfloat16, 81, K ** -0.5), rnd((M, N), torch.bfloat16, 82)
     gain = 1 + 0.1 * rnd((K,), torch.float32, 83)
     t = dict(rtol=2e-2, atol=2e-2)
     xn = ref.rmsnorm(x, gain, 1e-5).double()
-    torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), xn @ w.double().t(), **t)
+    normed = ops.linear(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()
+    torch.testing.assert_close(normed.double(), xn @ w.double().t(), **t)
     torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), residual=res.cuda()).cpu().double(),
                                x.double() @ w.double().t() + res.double(), **t)
     lg = ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32)          # the output table's case: 32-bit sums kept
-    assert lg.dtype == torch.float32 and ops._library_f32_out
+    assert lg.dtype == torch.float32
     torch.testing.assert_close(lg.cpu().double(), x.double() @ w.double().t(), rtol=1e-4, atol=1e-4)
     gu = (xn @ w.double().t()).to(torch.bfloat16).double()
     want = torch.nn.functional.silu(gu[:, 0::2]) * gu[:, 1::2]
     torch.testing.assert_close(ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), want,
                                rtol=3e-2, atol=3e-2)
+    if (N, K) not in ops.library_widths or M <= ops.few_rows:
+        # the few-row kernel: a row's result does not depend on its panel or on the other rows
+        for r in (0, M // 2, M - 1):
+            alone = ops.linear(x[r:r + 1].cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()
+            assert torch.equal(alone[0], normed[r])
 
 
-@pytest.mark.parametrize("M", [1, 4, 8, 9, 16, 17, 32])
+def test_library_product_at_listed_widths(ops_for):
+    """Every width that may go to the library's product (ops/library_widths.json), at row counts as serving brings
+    them: a few more than the few-row kernel takes, a portion beside decoded tokens, a prediction head's rows one
+    short of a portion. Each runs at the rounded row count of library_rows; the rows asked for are compared with
+    plain multiply-adds in 32-bit, and what lies behind the result's rows is the caller's and stays as it was."""
+    from tiny_inference_server_amd.ops.hip_ops import library_rows, _ptr
+    ops = ops_for(torch.bfloat16)
+    for i, (N, K) in enumerate(sorted(ops.library_widths)):
+        w = rnd((N, K), torch.bfloat16, 300 + i, K ** -0.5).cuda()
+        for M in (65, 200, 1024, 2047, 2112) + ((4096,) if i % 4 == 0 else ()):
+            x, res = rnd((M, K), torch.bfloat16, 400 + i).cuda(), rnd((M, N), torch.bfloat16, 500 + i).cuda()
+            print(f"library product: rows {M} (asked {library_rows(M)}), out {N}, in {K}", flush=True)
+            got = ops.linear(x, w, residual=res)
+            want, res32 = torch.empty(M, N, dtype=torch.float32, device="cuda"), res.float()
+            ops.gemm_plain.tis_gemm_plain(1, 0, _ptr(x), x.stride(0), _ptr(w), K, _ptr(res32), N, _ptr(want), N, M, N, K,
+                                          ops._stream())
+            torch.cuda.synchronize()
+            torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+            assert got.shape == (M, N) and ops._holds_rows(got, library_rows(M))
+    assert 0 < ops.gemm_library.cdll.tis_gemm_library_plans() <= 256
+
+
+@pytest.mark.parametrize("M", [1, 4, 8, 9, 16, 17, 32, 33, 48, 64])
 @pytest.mark.parametrize("N,K", [(96, 64), (1000, 96), (130, 264), (2304, 1536), (1536, 4096)])
 def test_skinny_product_with_fused_norm_residual_and_gate(ops_for, M, N, K):
     """The few-row matrix-core product and what is fused around it, against the unfused plain computation."""

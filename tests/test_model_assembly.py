@@ -96,7 +96,7 @@ def test_every_mixer_of_a_block_gets_a_cache_of_its_own_and_planning_comes_from_
                 super().__init__()
                 self.asked = []
 
-            def plan_attention(self, n_heads, n_kv_heads, head_dim, seq_rows, add, mode=None):
+            def plan_attention(self, n_heads, n_kv_heads, head_dim, seq_rows, add, mode=None, window=0):
                 self.asked.append((n_heads, n_kv_heads, head_dim))
                 return {("toy", n_heads): (add([1, 2, 3]), len(seq_rows))}
 

@@ -127,11 +127,11 @@ class PlanningOps(TorchOps):
     """The stand-in with the attention mixer's host planning switched on, as the real operations have it: the plan's
     arrays travel with the step, the stand-in's attention ignores them."""
 
-    def plan_attention_mode(self, seq_rows):
+    def plan_attention_mode(self, seq_rows, window=0):
         from tiny_inference_server_amd.ops.hip_ops import uneven_lengths
         return "uneven" if uneven_lengths(seq_rows) else None
 
-    def plan_attention(self, n_heads, n_kv_heads, head_dim, seq_rows, add, mode=None):
+    def plan_attention(self, n_heads, n_kv_heads, head_dim, seq_rows, add, mode=None, window=0):
         from tiny_inference_server_amd.ops.hip_ops import decode_items
         if mode != "uneven":
             return {}

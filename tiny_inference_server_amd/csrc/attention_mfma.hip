@@ -866,10 +866,25 @@ struct SideStream {
   hipEvent_t fork = nullptr, join = nullptr;
 };
 static SideStream g_side[64];
+static std::mutex g_side_mutex;      // set-up and launches may come from different threads
+
+// The second stream of the current device, as it was last set (a copy: the caller does not hold the lock).
+static SideStream side_of_current_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SideStream();
+  std::lock_guard<std::mutex> lock(g_side_mutex);
+  return g_side[dev];
+}
+
+// How many partial results a row and head may have: what both entry points size and lay out the workspace by.
+static int split_stride(int n_items, int n_tiles, int n_splits, int tile_splits) {
+  return std::max(n_items > 0 ? n_splits : 1, n_tiles > 0 ? tile_splits : 1);
+}
 
 TIS_EXPORT int tis_attention_mfma_side_stream(hipStream_t side) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return tis_fail("attention_mfma: no current device");
+  std::lock_guard<std::mutex> lock(g_side_mutex);
   SideStream& st = g_side[dev];
   if (side && !st.fork) {
     if (hipEventCreateWithFlags(&st.fork, hipEventDisableTiming) != hipSuccess ||
@@ -905,7 +920,7 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
   if (page_size < 16 || page_size % 16) return tis_fail("attention_mfma: page size %d is no multiple of 16", page_size);
   if (n_splits < 1 || n_splits > 65535 || tile_splits < 1 || tile_splits > 65535 || n_kv_heads > 65535)
     return tis_fail("attention_mfma: bad grid %d x %d (tiles: %d)", n_kv_heads, n_splits, tile_splits);
-  const int stride = n_splits > tile_splits ? n_splits : tile_splits;
+  const int stride = split_stride(n_items, n_tiles, n_splits, tile_splits);
   if (stride > 1 && (!part_o || !part_ml)) return tis_fail("attention_mfma: %d splits need a workspace", stride);
   if (min_steps < -1 || (min_steps == -1 && (!items || n_items < 1 || n_tiles > 0)))
     return tis_fail("attention_mfma: min_steps=%d; -1 goes with a planned list of single rows and no tiles", min_steps);
@@ -922,17 +937,20 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
   const float scale_log2 = scale * 1.4426950408889634f;
   int rc = 0;
   hipStream_t tile_stream = stream;
-  const SideStream* side = nullptr;
+  SideStream side;
+  bool forked = false;
   if (n_items > 0 && n_tiles > 0) {
-    int dev = 0;
-    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && g_side[dev].stream && g_side[dev].stream != stream) {
-      side = &g_side[dev];
+    side = side_of_current_device();
+    if (side.stream && side.stream != stream) {
       // the tiles wait for what came before this call, not for the items
-      if (hipEventRecord(side->fork, stream) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
-        return tis_fail("attention_mfma: the second stream could not be joined to the first");
-      tile_stream = side->stream;
+      if (hipEventRecord(side.fork, stream) != hipSuccess) return tis_fail("attention_mfma: the second stream could not be joined to the first");
+      if (hipStreamWaitEvent(side.stream, side.fork, 0) != hipSuccess) return tis_fail("attention_mfma: the second stream could not be joined to the first");
+      forked = true;
+      tile_stream = side.stream;
     }
   }
+  // From here on the second stream hangs off the first: whatever happens, it is joined again before this function
+  // returns, so that a stream capture never ends with a branch left open.
   if (n_items > 0) {
     dim3 grid(n_items, n_kv_heads, min_steps < 0 ? 1 : n_splits);
 #define LAUNCH(NBV, PSV)                                                                                              \
@@ -951,9 +969,8 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
     }
 #undef LAUNCH
     rc = tis_launch_status("attention_mfma");
-    if (rc) return rc;
   }
-  if (n_tiles > 0) {
+  if (n_tiles > 0 && rc == 0) {
     dim3 grid(n_tiles, n_kv_heads, tile_splits);
 #define LAUNCH(PSV)                                                                                                   \
   attention_tile_kernel<PSV><<<grid, TW * 64, 0, tile_stream>>>(                                                      \
@@ -964,11 +981,11 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
     else LAUNCH(false);
 #undef LAUNCH
     rc = tis_launch_status("attention_tile");
-    if (side && (hipEventRecord(side->join, side->stream) != hipSuccess ||
-                 hipStreamWaitEvent(stream, side->join, 0) != hipSuccess))
-      return tis_fail("attention_mfma: the first stream could not wait for the second");
-    if (rc) return rc;
   }
+  if (forked && (hipEventRecord(side.join, side.stream) != hipSuccess ||
+                 hipStreamWaitEvent(stream, side.join, 0) != hipSuccess))
+    return tis_fail("attention_mfma: the first stream could not wait for the second");
+  if (rc) return rc;
   if (stride > 1) {
     if ((long)rows * n_heads > 8192) {
       dim3 mgrid(rows, (n_heads + MG - 1) / MG);
@@ -1035,7 +1052,7 @@ TIS_EXPORT int tis_attention_mfma_static(const void* q, long q_ld, const void* p
   if ((n_items == 0 && n_tiles == 0) || rows == 0) return 0;
   if (rows < 0 || n_heads < 1 || n_splits < 1 || tile_splits < 1)
     return tis_fail("attention_mfma_static: bad sizes rows=%d heads=%d splits=%d, %d", rows, n_heads, n_splits, tile_splits);
-  const int stride = std::max(n_items > 0 ? n_splits : 1, n_tiles > 0 ? tile_splits : 1);
+  const int stride = split_stride(n_items, n_tiles, n_splits, tile_splits);
   float *part_o = nullptr, *part_ml = nullptr;
   int* row_splits = nullptr;
   if (stride > 1) {

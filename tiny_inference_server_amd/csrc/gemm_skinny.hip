@@ -1,5 +1,9 @@
-// C[M,N] = f(A[M,K]) . W[N,K]^T for few rows (M <= 32; 64 for the q/k/v projection): the matrix product of decode
-// steps, where the job is to stream W from HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950).
+// C[M,N] = f(A[M,K]) . W[N,K]^T for few rows: the matrix product of decode steps, where the job is to stream W from
+// HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950). A workgroup takes up to MB * 16 rows; more rows than that are cut
+// into panels of that many, one per blockIdx.y, each an independent product over the same weights (the panels of a
+// column tile run side by side, so the weights come from HBM once and from the caches after that). That is the right
+// kernel for a few panels; for many, every panel streams all of W again, which only a product tiled in both directions
+// avoids: it still gives the right result, slowly.
 //
 // One workgroup owns 16 rows of W (16 output columns; 8 in the narrow variant below) over the whole of K; its
 // waves take the 32-wide steps of K in turn, so together they read each weight row in contiguous runs. W rows are the A operand straight from
@@ -44,14 +48,16 @@ struct RopeArgs {
 
 // GS_WAVES: waves per workgroup; U: steps of K whose loads a wave issues together before the first product.
 // Eight waves of three or four steps measured best on MI355X for K of 1536 to 4096 (5.6 us for a 25 MB matrix,
-// 23 us for the 147 MB output table: 80 % of the HBM peak); four waves where K is too short to feed eight.
+// 23 us for the 147 MB output table: 80 % of the HBM peak); four waves where K is too short to feed eight. Batches
+// of eight steps, or sixteen waves, so that all of a wave's loads are in flight at once, measured the same within
+// noise (the gated product at 64 rows slower: fewer workgroups fit a compute unit).
 //
-// MB: blocks of 16 rows of X that share every weight tile a wave loads. Two blocks (17 to 32 rows) still beat the
-// library's product plus the separate norm, gate and rotary launches (7.8k against 6.4k tokens a second at batch
-// 20, 9.7k against 9.1k at batch 32); with four blocks the activations, which every workgroup reads in full from
-// L2, outweigh the weights four to one and the library wins (11.2k against 12.8k at batch 64), except for the
-// q/k/v projection, where this kernel stands for three launches (norm, product, rotary with cache write: 12.9k
-// against 12.7k at batch 64, 11.5k against 11.1k at batch 48); four blocks are built for that one only.
+// MB: blocks of 16 rows of X that share every weight tile a wave loads: one or two. More rows than 32 are further
+// panels (blockIdx.y): the panels of a column tile run side by side at the time of one (the down product, 12.6 MB:
+// 14.7 us at 32 rows, 14.6 at 64), which leaves this kernel ahead of the library's product with its separate norm,
+// gate and rotary launches up to 64 rows (whole decode steps at 0.9B, context 1,024, tokens a second, panels /
+// library: batch 48 17.9k / 16.4k, 64 21.4k / 20.3k, 96 24.0k / 24.1k, 128 26.7k / 29.7k). What a workgroup's time
+// goes to from 17 rows on is the activations: it reads all of its panel's X from L2 beside 16 rows of W.
 //
 // CT: column tiles of 16 a workgroup owns. Two where the matrix is so wide that half as many workgroups still fill
 // the chip: a wave then uses the activations it loaded (and normed) for twice as many weights.
@@ -76,6 +82,18 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
   const int chunk = c16 / COLS, sub = c16 % COLS;   // the lane's chunk of a step; its weight row and its activation row
   const int n0 = blockIdx.x * COLS * CT;
+  // the workgroup's panel of rows: everything below sees only these
+  {
+    const long m0 = (long)blockIdx.y * (MB * 16);
+    X += m0 * x_ld;
+    C += m0 * c_ld;
+    if (EPI == EPI_RESIDUAL) R_in += m0 * r_ld;
+    if (EPI == EPI_ROPE) {
+      rope.positions += m0;
+      if (rope.write_slots) rope.write_slots += m0;
+    }
+    M = min(M - (int)m0, MB * 16);
+  }
   const int steps = (K + 32 * R - 1) / (32 * R);
   bool w_ok[CT];
   const bf16* wrow[CT];
@@ -283,9 +301,10 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
   }
 }
 
-// (both can be set from outside: the kernel tests make small matrices take the wide path)
+// (these can be set from outside: the kernel tests make small matrices take the wide path, and measurements compare
+// panel heights)
 static int g_wide_tiles = 256;   // from this many 32-column workgroups on (one a compute unit), a workgroup takes two column tiles
-static int g_wide_max_blocks = 2;   // with up to two blocks of 16 rows (four blocks measured no gain over the library)
+static int g_wide_max_blocks = 2;   // with up to two blocks of 16 rows
 TIS_EXPORT void tis_gemm_skinny_wide_tiles(int n_workgroups) { g_wide_tiles = n_workgroups; }
 TIS_EXPORT void tis_gemm_skinny_wide_max_blocks(int n) { g_wide_max_blocks = n; }
 
@@ -299,7 +318,10 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
   int r = (M <= 8 && (N + 15) / 16 <= 128) ? 2 : 1;
   if (r != 1 && r != 2) return tis_fail("gemm_skinny: %d chunks a step; 1 or 2 are built", r);
   if (r == 2 && M > 8) return tis_fail("gemm_skinny: %d rows do not fit 8 columns a workgroup", M);
-  const int mb = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+  // rows beyond a panel's go to further panels (blockIdx.y)
+  const int mb = M <= 16 ? 1 : 2;
+  const int panels = (M + mb * 16 - 1) / (mb * 16);
+  if (panels > 65535) return tis_fail("gemm_skinny: %d rows are more panels than a grid holds", M);
   const int steps = (K + 32 * r - 1) / (32 * r);
   int waves, u;
   if (steps >= 24) {
@@ -310,7 +332,7 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
     waves = 4;
     u = (steps % 3 == 0 && steps % 4 != 0) || steps == 12 ? 3 : 4;
   }
-  if (mb > 1 && waves != 8) { waves = 8; u = 4; }   // several row blocks are built for eight waves only
+  if (mb > 1 && waves != 8) { waves = 8; u = 4; }   // two row blocks are built for eight waves only
   // two column tiles a workgroup where the matrix is wide enough to fill the chip with half as many workgroups:
   // the activations, the gains and the norm's arithmetic are then shared by twice as many weights (the gate-up
   // product of 8192 columns and the output table: 2.5 % of a decode step at batch 8)
@@ -319,11 +341,11 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
     if (r == 1 && mb <= g_wide_max_blocks && waves == 8 && (N + 31) / 32 >= g_wide_tiles) ct = 2;
   }
   const int cols = 16 / r * ct;
-  const int n_wg = (N + cols - 1) / cols;
+  const dim3 grid((N + cols - 1) / cols, panels);
   if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) {
 #define WIDE(MBV, UV)                                                                                            \
   if (ct == 2 && mb == MBV && u == UV) {                                                                         \
-    gemm_skinny_kernel<MBV, NORM, EPI, TO, 8, UV, 1, 2><<<n_wg, 8 * 64, 0, stream>>>(                            \
+    gemm_skinny_kernel<MBV, NORM, EPI, TO, 8, UV, 1, 2><<<grid, 8 * 64, 0, stream>>>(                            \
         (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);     \
     return 0;                                                                                                    \
   }
@@ -332,14 +354,13 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
   }
 #define CFG(MBV, WV, UV, RV)                                                                                     \
   if (ct == 1 && mb == MBV && waves == WV && u == UV && r == RV) {                                               \
-    gemm_skinny_kernel<MBV, NORM, EPI, TO, WV, UV, RV, 1><<<n_wg, WV * 64, 0, stream>>>(                         \
+    gemm_skinny_kernel<MBV, NORM, EPI, TO, WV, UV, RV, 1><<<grid, WV * 64, 0, stream>>>(                         \
         (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);     \
     return 0;                                                                                                    \
   }
 #define CFGS(RV) CFG(1, 4, 3, RV) CFG(1, 4, 4, RV) CFG(1, 8, 3, RV) CFG(1, 8, 4, RV)
   CFGS(1) CFGS(2)
   CFG(2, 8, 3, 1) CFG(2, 8, 4, 1)
-  if constexpr (EPI == EPI_ROPE) { CFG(4, 8, 3, 1) CFG(4, 8, 4, 1) }   // four blocks: built for the q/k/v projection only
 #undef CFGS
 #undef CFG
   return tis_fail("gemm_skinny: no kernel for %d row blocks, %d waves of %d steps and %d chunks", mb, waves, u, r);
@@ -357,7 +378,7 @@ TIS_EXPORT int tis_gemm_skinny(const void* X, long x_ld, const void* W, const fl
                                long r_ld, void* C, long c_ld, int M, int N, int K, int epilogue, int out_dtype,
                                hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
-  if (M < 0 || M > 32) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..32", M);
+  if (M < 0) return tis_fail("gemm_skinny: %d rows", M);
   if (N < 1 || K < 8 || K % 8) return tis_fail("gemm_skinny: N=%d K=%d; K must be a multiple of 8", N, K);
   if (x_ld % 8 || ((uintptr_t)X % 16) || ((uintptr_t)W % 16))
     return tis_fail("gemm_skinny: activations and weights must be 16-byte aligned with row strides in steps of 8");
@@ -383,7 +404,7 @@ TIS_EXPORT int tis_gemm_skinny_qkv_rope(const void* X, long x_ld, const void* W,
                                         const float* table, void* plane, int n_heads, int n_kv_heads, int head_dim,
                                         int page_size, int interleaved, int write_cache, hipStream_t stream) {
   if (M == 0) return 0;
-  if (M < 0 || M > 64) return tis_fail("gemm_skinny: %d rows; this kernel takes 1..64", M);
+  if (M < 0) return tis_fail("gemm_skinny: %d rows", M);
   if (K < 8 || K % 8) return tis_fail("gemm_skinny: K=%d must be a multiple of 8", K);
   if (n_heads < 1 || n_kv_heads < 1 || head_dim < 4 || head_dim % 4 || page_size < 1)
     return tis_fail("gemm_skinny: heads=%d kv_heads=%d head_dim=%d (a multiple of 4) page=%d", n_heads, n_kv_heads,

@@ -257,7 +257,7 @@ class Engine:
         head_logits = head_valid = None
         if logits is None:
             if heads and len(outs) > 1:
-                logits, head_logits, head_valid = self._all_logits(outs, n)
+                logits, head_logits, head_valid = self.model.logits_of_stages(outs, n)
             else:
                 logits = self.logits_of(outs, step, n)
         windows = self._has_windows
@@ -277,34 +277,6 @@ class Engine:
         if n:
             return self.model.logits(outs[0].hidden, step.stages[0].want_index, n)
         return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
-
-    def _all_logits(self, outs, n):
-        """Logits of every stage at the wanted places from one product with the output table, which all stages share
-        (reference main_models_new.py:225-226): the table is read once however many stages there are. Rows that a
-        prediction stage does not have yet come back as NaN."""
-        vocab, S = self.spec.vocab_size, len(outs)
-        if n == 0:
-            e = torch.empty(0, vocab, dtype=torch.float32, device=self.device)
-            return e, [e.clone() for _ in outs[1:]], [[] for _ in outs[1:]]
-        rows = self.ops.empty(S * n, self.spec.d_model)
-        valid = []
-        for j, o in enumerate(outs):
-            v = [True] * n if j == 0 else list(o.batch.want_valid)
-            part = rows[j * n:(j + 1) * n]
-            if o.batch.n_rows and any(v):
-                idx = o.batch.want_index[:n] if j == 0 else torch.clamp(o.batch.want_index[:n], min=0)
-                self.ops.gather_rows(o.hidden, o.hidden, idx, out=part)
-            else:
-                part.zero_()
-            valid.append(v)
-        lg = self.ops.linear(rows, self.model.shared["lm_head"], out_dtype=torch.float32).view(S, n, vocab)
-        head_logits = []
-        for j in range(1, S):
-            h = lg[j]
-            if not all(valid[j]):
-                h[~torch.tensor(valid[j], device=self.device)] = float("nan")
-            head_logits.append(h)
-        return lg[0], head_logits, valid[1:]
 
     def _make_room(self, of_kind, limit: int) -> None:
         """Drop the least recently used graphs of one kind until another fits under `limit`."""

@@ -145,7 +145,43 @@ class Model:
                 after(step.stages[j], hidden[j - 1], cache.states.get(self.state_keys[j]) if self.state_keys[j] else None)
         return [StageOutput(hidden[j], step.stages[j]) for j in range(n)]
 
+    def _wanted_rows(self, hidden, want_index, n, out=None):
+        return self.ops.gather_rows(hidden, hidden, want_index[:n], out=out)
+
+    def _project(self, rows):
+        """Rows after a stage's closing norm -> 32-bit logits: the one place the output table is applied."""
+        return self.ops.linear(rows, self.shared["lm_head"], out_dtype=torch.float32)
+
     def logits(self, hidden, want_index, n):
         """32-bit logits [n, vocab] of the rows `want_index` of `hidden` (reference main_models_new.py:225-226)."""
-        rows = self.ops.gather_rows(hidden, hidden, want_index[:n])
-        return self.ops.linear(rows, self.shared["lm_head"], out_dtype=torch.float32)
+        return self._project(self._wanted_rows(hidden, want_index, n))
+
+    def logits_of_stages(self, outs, n):
+        """Logits of every stage at the n wanted places from one product with the output table, which all stages
+        share (reference main_models_new.py:225-226): the table is read once however many stages there are.
+        Returns (first stage's logits [n, vocab], [logits of each further stage], [which of their rows are valid]);
+        rows that a later stage does not have yet come back as NaN. The first stage's part equals `logits` bit for
+        bit: same gather, same product, a row's result does not depend on the other rows."""
+        vocab, S = self.spec.vocab_size, len(outs)
+        if n == 0:
+            e = torch.empty(0, vocab, dtype=torch.float32, device=self.ops.device)
+            return e, [e.clone() for _ in outs[1:]], [[] for _ in outs[1:]]
+        rows = self.ops.empty(S * n, self.spec.d_model)
+        valid = []
+        for j, o in enumerate(outs):
+            v = [True] * n if j == 0 else list(o.batch.want_valid)
+            part = rows[j * n:(j + 1) * n]
+            if o.batch.n_rows and any(v):
+                idx = o.batch.want_index[:n] if j == 0 else torch.clamp(o.batch.want_index[:n], min=0)
+                self._wanted_rows(o.hidden, idx, n, out=part)
+            else:
+                part.zero_()
+            valid.append(v)
+        lg = self._project(rows).view(S, n, vocab)
+        later = []
+        for j in range(1, S):
+            h = lg[j]
+            if not all(valid[j]):
+                h[~torch.tensor(valid[j], device=self.ops.device)] = float("nan")
+            later.append(h)
+        return lg[0], later, valid[1:]

@@ -6,10 +6,18 @@ libraries construction fails. Matrix products in bfloat16 of a few rows go to th
 (csrc/gemm_skinny.hip), those of many rows to hipBLASLt through csrc/gemm_library.hip, as the reference's go to
 a library (main_models_new.py:19-20); in 32-bit they go to the plain multiply-add kernel so that no
 reduced-precision matrix mode can take part.
+
+The library is only ever asked for products whose widths (output columns, input columns) stand in
+ops/library_widths.json, the list of widths that this repository's GPU tests and benchmarks run, and only at row
+counts from one family (library_rows): a library kernel differs from shape to shape, and a shape that nothing has
+run is a kernel that nothing has tested. Any other product runs on this repository's own kernels: right at every
+size, slower where there are many rows.
 """
 from __future__ import annotations
 
 import ctypes
+import json
+import os
 from ctypes import c_float, c_int, c_long, c_void_p
 from typing import NamedTuple, Optional
 
@@ -102,11 +110,41 @@ def library(name: str) -> _Lib:
     return lib
 
 
+_FEW_ROWS = 64                  # up to this many rows a product goes to the few-row kernel whatever its widths
+
+_WIDTHS_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "library_widths.json")
+
+
+def library_widths(path: str = _WIDTHS_FILE):
+    """The (output columns, input columns) pairs that may go to the library's product: a data file, not code."""
+    with open(path) as f:
+        return frozenset((int(n), int(k)) for n, k in json.load(f)["widths"])
+
+
+def library_rows(m: int) -> int:
+    """The row count the library is asked for when a product has `m` rows: the next multiple of 64 up to 256 rows,
+    of 256 beyond. A serving run's steps bring row counts that nobody chose (a portion beside some decoded tokens, a
+    prediction head's rows one short of the trunk's); rounded up, they all become the few shapes that every
+    benchmark and test of a width has already run. The extra rows are computed on whatever lies behind the operands'
+    rows and are never read."""
+    step = 64 if m <= 256 else 256
+    return -(-m // step) * step
+
+
+def product_route(M: int, N: int, K: int, aligned: bool, out_f32: bool, widths, few_rows: int = _FEW_ROWS):
+    """Which kernel takes a bfloat16 product of M rows, N output and K input columns: "few_rows" (the fused few-row
+    kernel, in panels of rows beyond its own height), "library" (at library_rows(M) rows) or "plain" (multiply-adds,
+    for operands that do not lie as the other two need them). Pure: the decision can be checked without a device."""
+    if not aligned:
+        return "plain"
+    if M <= few_rows or out_f32 or (N, K) not in widths:
+        return "few_rows"
+    return "library"
+
+
 # wavefronts the attention launch aims for, so that short batches still spread over the chip
-_SKINNY_MAX_ROWS = 32
-_SKINNY_MAX_ROWS_QKV = 64        # the q/k/v projection with norm, rotary and cache write fused stands for three launches
 _ATTN_TARGET_WAVES = 512
-_CHIP_UNITS = 256               # compute units of an MI355X
+_CHIP_UNITS = 256               # compute units of an MI355X: the default where no device is asked (host-only tests)
 _ATTN_PROMPT_TARGET_WAVES = 2048  # what the grid offers where rows of prompts are in the batch ...
 _ATTN_PROMPT_SPLIT_MAX_ROWS = 512 # ... and the batch is small; a long portion fills the chip by its rows alone
 _ATTN_PROMPT_MIN_STEPS = 8         # steps of 32 keys below which a prompt item's split is not worth its merge
@@ -198,9 +236,10 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
     return nb, cut(rest, max(1, (16 * nb) // group_size))[0], tiles, steps
 
 
-def uneven_lengths(seq_rows) -> bool:
+def uneven_lengths(seq_rows, window: int = 0) -> bool:
     """Whether a step of single rows holds requests of such different lengths that equal split counts would leave the
-    longest request's waves running on alone: then the splits are planned request by request (decode_items)."""
+    longest request's waves running on alone: then the splits are planned request by request (decode_items). With a
+    window a row's length is what it sees of its request."""
     n = len(seq_rows)
     if n < 2:
         return False
@@ -208,7 +247,7 @@ def uneven_lengths(seq_rows) -> bool:
     for _, p0, rows in seq_rows:            # (one pass: this runs for every step of decoded tokens)
         if rows != 1:
             return False
-        steps = (p0 + 32) >> 5
+        steps = (p0 + 32) >> 5 if window <= 0 or p0 < window else (p0 + 32 - ((p0 - window + 1) & ~31)) >> 5
         total += steps
         if steps > longest:
             longest = steps
@@ -220,15 +259,15 @@ def planned_list_pays(n_rows: int, n_kv_heads: int) -> bool:
     return n_rows >= _ATTN_PLANNED_MIN_ROWS and n_rows * n_kv_heads <= _ATTN_PLANNED_MAX_WAVES
 
 
-def planned_target_waves(n_kv_heads: int) -> int:
-    return max(_ATTN_TARGET_WAVES, _CHIP_UNITS * n_kv_heads)
+def planned_target_waves(n_kv_heads: int, units: int = _CHIP_UNITS) -> int:
+    return max(_ATTN_TARGET_WAVES, units * n_kv_heads)
 
 
-def decode_items_capacity(n_rows: int, n_kv_heads: int) -> int:
+def decode_items_capacity(n_rows: int, n_kv_heads: int, units: int = _CHIP_UNITS) -> int:
     """Entries of a planned list for `n_rows` single rows: what the splits can add up to, whatever the lengths."""
     # (a multiple of the eight XCDs: workgroups go to them in turn, so the waves of an entry's key/value heads, which
     # read the same pages, then meet in one L2: 162 against 183 us at 8 key/value heads)
-    return -(-(planned_target_waves(n_kv_heads) // n_kv_heads + n_rows + 1) // 8) * 8
+    return -(-(planned_target_waves(n_kv_heads, units) // n_kv_heads + n_rows + 1) // 8) * 8
 
 
 def decode_items_most_splits(n_rows: int, n_heads: int, head_dim: int, workspace_floats=None) -> int:
@@ -237,7 +276,8 @@ def decode_items_most_splits(n_rows: int, n_heads: int, head_dim: int, workspace
     return int(max(1, min(_ATTN_DECODE_MAX_SPLITS, (workspace_floats - n_rows) // (n_rows * n_heads * (head_dim + 2)))))
 
 
-def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspace_floats=None):
+def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspace_floats=None, window: int = 0,
+                 units: int = _CHIP_UNITS):
     """The work list of a step of single rows whose requests differ widely in length: one entry per wave (and
     key/value head), (row, split + 65536 * splits of the row, position, block-table line), so that every wave walks
     about the same number of keys; longest first; padded with row -1 to a length that depends on the number of rows
@@ -245,12 +285,15 @@ def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspa
     n = len(seq_rows)
     rows = np.fromiter((f for f, _, _ in seq_rows), dtype=np.int64, count=n)
     pos = np.fromiter((p0 for _, p0, _ in seq_rows), dtype=np.int64, count=n)
-    steps = (pos + 32) // 32                                     # a row at position p sees p + 1 keys
+    # a row at position p sees p + 1 keys, or the last `window` of them; the kernel walks them in steps of 32 from a
+    # multiple of 32
+    first = np.maximum(0, pos - window + 1) & ~31 if window > 0 else 0
+    steps = (pos + 32 - first) // 32
     fewest = max(1, _ATTN_MIN_SPLIT_KEYS // 32)
-    even = max(fewest, -(-int(steps.sum()) * n_kv_heads // planned_target_waves(n_kv_heads)))
+    even = max(fewest, -(-int(steps.sum()) * n_kv_heads // planned_target_waves(n_kv_heads, units)))
     most = decode_items_most_splits(n, n_heads, head_dim, workspace_floats)
     splits = np.clip((steps + even // 2) // even, 1, np.minimum(steps, most))
-    cap = decode_items_capacity(n, n_kv_heads)
+    cap = decode_items_capacity(n, n_kv_heads, units)
     total = int(splits.sum())
     if total > cap:
         raise KernelError(f"attention: {total} planned splits for a list of {cap}")
@@ -284,7 +327,7 @@ class AttentionLaunch(NamedTuple):
 
 
 def attention_launch_plan(n, n_items, n_tiles, tile_steps, single, max_kv_len, n_heads, n_kv_heads, head_dim,
-                          workspace_floats=None, planned_splits=0) -> AttentionLaunch:
+                          workspace_floats=None, planned_splits=0, units: int = _CHIP_UNITS) -> AttentionLaunch:
     """Split counts of one attention call over `n` rows, from the planner's items and tiles; pure host arithmetic.
     planned_splits > 0: the items are a list planned by decode_items, whose rows have at most that many splits."""
     workspace_floats = _ATTN_WORKSPACE_FLOATS if workspace_floats is None else workspace_floats
@@ -306,7 +349,7 @@ def attention_launch_plan(n, n_items, n_tiles, tile_steps, single, max_kv_len, n
             # 79 us, 3 splits 82; 32 requests: 8 splits 37, 6 splits 40; at 8,192 keys 146 against 163)
             waves = n_items * n_kv_heads
             for s in range(n_splits, min(2 * n_splits, max_kv_len // min_keys) + 1):
-                if waves * s % _CHIP_UNITS == 0:
+                if waves * s % units == 0:
                     n_splits = s
                     break
         min_steps = 0 if single else _ATTN_PROMPT_MIN_STEPS
@@ -374,7 +417,11 @@ class HipOps:
         self.sampling = library("sampling")
         self.gemm_skinny = library("gemm_skinny") if dtype == torch.bfloat16 else None
         self.gemm_library = None
-        self._library_f32_out = True
+        self.few_rows = _FEW_ROWS
+        self.library_widths = library_widths()
+        self._warned_widths = set()
+        # compute units of this device: what the attention planner spreads waves over
+        self.units = int(torch.cuda.get_device_properties(self.device).multi_processor_count) or _CHIP_UNITS
         if dtype == torch.bfloat16:
             self.gemm_library = library("gemm_library")
             with torch.cuda.device(self.device):
@@ -385,12 +432,13 @@ class HipOps:
             if dtype == torch.bfloat16 else None
 
     # ---- planning on the host --------------------------------------------------------------------------
-    def plan_attention_mode(self, seq_rows):
+    def plan_attention_mode(self, seq_rows, window: int = 0):
         """What kind of plan a step gets, from its first stage's rows: two steps may share a captured graph only if
-        this is equal. "uneven": single rows of requests that differ widely in length."""
-        return "uneven" if self.dtype == torch.bfloat16 and uneven_lengths(seq_rows) else None
+        this is equal. "uneven": single rows of requests that differ widely in length (in what a row sees of its
+        request, where the mixer has a window)."""
+        return "uneven" if self.dtype == torch.bfloat16 and uneven_lengths(seq_rows, window) else None
 
-    def plan_attention(self, n_heads: int, n_kv_heads: int, head_dim: int, seq_rows, add, mode=None):
+    def plan_attention(self, n_heads: int, n_kv_heads: int, head_dim: int, seq_rows, add, mode=None, window: int = 0):
         """An attention mixer's host planning, called while a step's arrays are packed: the work items of the
         matrix-core kernels for the step's rows. Returns {name: (packed array id, host values...)}."""
         plans = {}
@@ -398,12 +446,13 @@ class HipOps:
             group, cols = n_heads // n_kv_heads, tile_columns(head_dim)
             if (mode == "uneven" and group <= 64 and planned_list_pays(len(seq_rows), n_kv_heads)
                     and all(n == 1 for _, _, n in seq_rows)):
-                entries, most = decode_items(seq_rows, n_heads, n_kv_heads, head_dim)
-                return {("attention_decode_items", group, cols, n_kv_heads): (add(entries), len(entries), most)}
+                entries, most = decode_items(seq_rows, n_heads, n_kv_heads, head_dim, window=window, units=self.units)
+                return {("attention_decode_items", group, cols, n_kv_heads, window): (add(entries), len(entries), most)}
             nb, items, tiles, steps = attention_items(seq_rows, group, cols, n_kv_heads)
             if nb <= 4 and (len(items) or len(tiles)):
                 # one array: the items' lines, then the tiles'
-                plans[("attention_items", group, cols, n_kv_heads)] = (add(np.concatenate((items, tiles))), len(items),
+                # (a mixer with a window plans for itself: its lists are the same, its keys are its own)
+                plans[("attention_items", group, cols, n_kv_heads, window)] = (add(np.concatenate((items, tiles))), len(items),
                                                                        nb, len(tiles), steps)
         return plans
 
@@ -431,7 +480,15 @@ class HipOps:
         return t
 
     def empty(self, *shape, dtype=None):
-        return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)
+        """An uninitialised tensor. Rows of bfloat16 activations that may go into the library's product are allocated
+        up to the row count the library is asked for (library_rows), so that the product can run on them as they
+        lie; the tensor that comes back shows the rows asked for."""
+        dtype = dtype or self.dtype
+        if len(shape) == 2 and dtype == torch.bfloat16 and shape[0] > self.few_rows:
+            rows = library_rows(shape[0])
+            if rows != shape[0]:
+                return torch.empty(rows, shape[1], dtype=dtype, device=self.device)[:shape[0]]
+        return torch.empty(*shape, dtype=dtype, device=self.device)
 
     # ---- row-wise ------------------------------------------------------------------------------------
     def embedding(self, table, tokens, out=None):
@@ -529,8 +586,8 @@ class HipOps:
         """f(x)[M,K] . w[N,K]^T (+ residual[M,N]); `out_dtype` float32 gives 32-bit results from bfloat16 inputs.
 
         rms = (gain, eps): f is the RMSNorm of the rows, fused into the product where the kernel allows.
-        reuse_residual: the caller has no further use for `residual`, so the result may be written over it
-        (the library's product then adds in place instead of copying the residual first).
+        reuse_residual: the caller has no further use for `residual`; an operations object may then write the result
+        over it. This one never does: every product's result has memory of its own.
         """
         _rows_view(self._check(x, "linear x"), "linear x")
         self._check(w, "linear w")
@@ -547,36 +604,59 @@ class HipOps:
             self._check(rms[0], "rmsnorm gain", torch.float32)
             if rms[0].numel() != K or not rms[0].is_contiguous():
                 raise KernelError(f"linear: norm gain has {rms[0].numel()} entries for width {K}")
-        if self._skinny_ok(x, M, K):
-            out = self.empty(M, N, dtype=out_dtype)
-            self.gemm_skinny.tis_gemm_skinny(
-                _ptr(x), x.stride(0), _ptr(w), _ptr(rms[0] if rms else None), float(rms[1]) if rms else 0.0,
-                _ptr(residual), residual.stride(0) if residual is not None else 0, _ptr(out), N, M, N, K,
-                1 if residual is not None else 0, _DT[out_dtype], self._stream())
-            return out
-        if rms is not None:
-            x = self.rmsnorm(x, rms[0], rms[1])
         if self.dtype == torch.float32:
+            if rms is not None:
+                x = self.rmsnorm(x, rms[0], rms[1])
             out = self.empty(M, N, dtype=torch.float32)
             self.gemm_plain.tis_gemm_plain(0, 0, _ptr(x), x.stride(0), _ptr(w), K, _ptr(residual),
                                            residual.stride(0) if residual is not None else 0, _ptr(out), N, M, N, K,
                                            self._stream())
             return out
-        return self._linear_bf16(x, w, residual, out_dtype, reuse_residual)
+        route = self._route(x, M, N, K, out_dtype, residual)
+        if route == "few_rows":
+            out = self.empty(M, N, dtype=out_dtype)
+            if out_dtype == torch.float32 and residual is not None:
+                raise KernelError("linear: a 32-bit result of bfloat16 operands takes no residual")
+            self.gemm_skinny.tis_gemm_skinny(
+                _ptr(x), x.stride(0), _ptr(w), _ptr(rms[0] if rms else None), float(rms[1]) if rms else 0.0,
+                _ptr(residual), residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0), M, N, K,
+                1 if residual is not None else 0, _DT[out_dtype], self._stream())
+            return out
+        if rms is not None:
+            x = self.rmsnorm(x, rms[0], rms[1])
+        if route == "library":
+            return self._linear_library(x, w, residual)
+        out = self.empty(M, N, dtype=out_dtype)
+        self.gemm_plain.tis_gemm_plain(1, _DT[out_dtype], _ptr(x), x.stride(0), _ptr(w), K, _ptr(residual),
+                                       residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0), M, N,
+                                       K, self._stream())
+        return out
 
-    def _skinny_ok(self, x, M, K, limit=None):
-        # up to 32 rows the fused few-row kernel wins (it saves the norm, gating and rotary launches and streams the
-        # weights as fast as the library does); beyond, the library's product is enough faster to pay for them
-        return (self.dtype == torch.bfloat16 and 0 < M <= (limit or _SKINNY_MAX_ROWS) and K % 8 == 0 and x.stride(0) % 8 == 0
-                and x.data_ptr() % 16 == 0)
+    def _route(self, x, M, N, K, out_dtype=None, residual=None):
+        """Which kernel takes this bfloat16 product (see product_route); says once per width that a product of many
+        rows runs on the few-row kernel because the library's list does not hold its widths."""
+        aligned = K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+        route = product_route(M, N, K, aligned, out_dtype == torch.float32, self.library_widths, self.few_rows)
+        if route == "library" and residual is not None and (residual.stride(0) % 8 or residual.data_ptr() % 16):
+            route = "few_rows"
+        if route == "few_rows" and M > 8 * self.few_rows and (N, K) not in self._warned_widths \
+                and out_dtype != torch.float32:
+            self._warned_widths.add((N, K))
+            print(f"[tis-amd] a product of {M} rows with {N} output and {K} input columns runs on the few-row kernel: "
+                  f"these widths are not in {os.path.basename(_WIDTHS_FILE)} (the widths the library's product has "
+                  f"been tested at)", file=__import__("sys").stderr, flush=True)
+        return route
+
+    def _few_rows_ok(self, x, M, N, K):
+        return self.dtype == torch.bfloat16 and M > 0 and self._route(x, M, N, K) == "few_rows"
 
     def linear_swiglu(self, x, w, rms=None):
         """silu(g) * u of the rows of f(x) . w^T, w holding gate and up rows interleaved: [M, N/2]."""
         _rows_view(self._check(x, "linear x"), "linear x")
         M, K = x.shape
-        if self._skinny_ok(x, M, K) and w.shape[0] % 2 == 0:
+        if w.dim() == 2 and w.shape[0] % 2 == 0 and self._few_rows_ok(x, M, w.shape[0], K):
             self._check(w, "linear w")
-            if w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+            if w.shape[1] != K or not w.is_contiguous():
                 raise KernelError(f"linear: x {tuple(x.shape)} against w {tuple(w.shape)} (w is [out, in], contiguous)")
             if rms is not None and (rms[0].numel() != K or rms[0].dtype != torch.float32):
                 raise KernelError(f"linear: norm gain has {rms[0].numel()} entries for width {K}")
@@ -584,36 +664,42 @@ class HipOps:
             out = self.empty(M, N // 2)
             self.gemm_skinny.tis_gemm_skinny(
                 _ptr(x), x.stride(0), _ptr(w), _ptr(rms[0] if rms else None), float(rms[1]) if rms else 0.0,
-                _ptr(None), 0, _ptr(out), N // 2, M, N, K, 2, 1, self._stream())
+                _ptr(None), 0, _ptr(out), out.stride(0), M, N, K, 2, 1, self._stream())
             return out
         return self.swiglu(self.linear(x, w, rms=rms))
 
-    def _linear_bf16(self, x, w, residual, out_dtype, reuse_residual=False):
-        """The library's product for many rows (reference main_models_new.py:19-20 uses one too)."""
+    @staticmethod
+    def _holds_rows(t, rows: int) -> bool:
+        """Whether `rows` rows of t's stride lie inside the memory behind t."""
+        last = t.storage_offset() + (rows - 1) * t.stride(0) + t.shape[1]
+        return last * t.element_size() <= t.untyped_storage().nbytes()
+
+    def _with_rows(self, t, rows: int):
+        """t itself if the memory behind it holds `rows` rows (tensors from `empty` do), else a copy that does."""
+        if self._holds_rows(t, rows):
+            return t
+        c = self.empty(t.shape[0], t.shape[1], dtype=t.dtype)
+        c.copy_(t)
+        return c
+
+    def _linear_library(self, x, w, residual):
+        """The library's product for many rows (reference main_models_new.py:19-20 uses one too), asked at
+        library_rows(M) rows: the operands' memory reaches that far, and the rows beyond M are not looked at again.
+        The result has memory of its own, also where the caller has no further use for the residual."""
         M, K = x.shape
         N = w.shape[0]
-        aligned = not (x.stride(0) % 8 or x.data_ptr() % 16 or
-                       (residual is not None and (residual.stride(0) % 8 or residual.data_ptr() % 16)))
-        if out_dtype == torch.float32:
-            if aligned and residual is None and self._library_f32_out:
-                out = self.empty(M, N, dtype=torch.float32)      # 32-bit sums written as they are, not via bfloat16
-                try:
-                    self.gemm_library.tis_gemm_library(_ptr(x), x.stride(0), _ptr(w), _ptr(None), 0, _ptr(out), N, M, N,
-                                                       K, 1, self._stream())
-                    return out
-                except KernelError:
-                    self._library_f32_out = False       # a library without such kernels: round through bfloat16 below
-            out = torch.matmul(x, w.t()).float()
-            if residual is not None:
-                out += residual
-            return out
-        if not aligned:
-            # operands the library's fast kernels may not take as they lie: let the framework arrange them
-            return torch.addmm(residual, x, w.t()) if residual is not None else torch.matmul(x, w.t())
-        out = residual if (residual is not None and reuse_residual) else self.empty(M, N)
+        rows = library_rows(M)
+        if (N, K) not in self.library_widths:
+            raise KernelError(f"linear: widths ({N}, {K}) are not among those the library's product is used at")
+        x = self._with_rows(x, rows)
+        if residual is not None:
+            residual = self._with_rows(residual, rows)
+        out = self.empty(M, N)
+        if not self._holds_rows(out, rows):
+            raise KernelError(f"linear: the result of {M} rows has no room for {rows}")
         self.gemm_library.tis_gemm_library(_ptr(x), x.stride(0), _ptr(w), _ptr(residual),
                                            residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0),
-                                           M, N, K, 0, self._stream())
+                                           rows, N, K, 0, self._stream())
         return out
 
     # ---- position encoding + cache write, attention --------------------------------------------------
@@ -663,7 +749,7 @@ class HipOps:
         N = (n_heads + 2 * n_kv_heads) * head_dim
         if w.dim() != 2 or tuple(w.shape) != (N, K) or not w.is_contiguous():
             raise KernelError(f"qkv_rope: w {tuple(w.shape)} is not [{N}, {K}] contiguous")
-        if self._skinny_ok(x, M, K, _SKINNY_MAX_ROWS_QKV) and head_dim % 4 == 0:
+        if self._few_rows_ok(x, M, N, K) and head_dim % 4 == 0:
             self._index(positions, "positions", M)
             if table is not None:
                 self._check(table, "rotary table", torch.float32)
@@ -730,12 +816,13 @@ class HipOps:
         if (slopes is None and self.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 16 == 0
                 and group <= 64 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0):
             cols = tile_columns(head_dim)
-            planned = batch.extras.get(("attention_decode_items", group, cols, n_kv_heads))
-            plan = batch.extras.get(("attention_items", group, cols, n_kv_heads))
+            planned = batch.extras.get(("attention_decode_items", group, cols, n_kv_heads, int(window)))
+            plan = batch.extras.get(("attention_items", group, cols, n_kv_heads, int(window)))
             if planned is None and plan is None:
                 # a caller that did not plan (a kernel test): plan now, tiles wherever they fit
-                if uneven_lengths(batch.seq_rows) and planned_list_pays(n, n_kv_heads):
-                    entries, most = decode_items(batch.seq_rows, n_heads, n_kv_heads, head_dim)
+                if uneven_lengths(batch.seq_rows, int(window)) and planned_list_pays(n, n_kv_heads):
+                    entries, most = decode_items(batch.seq_rows, n_heads, n_kv_heads, head_dim, window=int(window),
+                                                 units=self.units)
                     planned = (torch.from_numpy(entries).reshape(-1).to(self.device), len(entries), most)
                 else:
                     nb, host_items, host_tiles, steps = attention_items(batch.seq_rows, group, cols)
@@ -770,7 +857,7 @@ class HipOps:
                                       f"assumes {cols}")
             single = items is None and n_tiles == 0
             lp = attention_launch_plan(n, n_items, n_tiles, tile_steps, single, batch.max_kv_len, n_heads, n_kv_heads,
-                                       head_dim, planned_splits=planned_splits)
+                                       head_dim, planned_splits=planned_splits, units=self.units)
             n_splits, min_steps, tile_splits, tile_max_steps = lp.n_splits, lp.min_steps, lp.tile_splits, lp.tile_max_steps
             part_o = part_ml = row_splits = None
             if lp.stride > 1:

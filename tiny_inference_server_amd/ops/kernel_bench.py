@@ -76,13 +76,13 @@ def attention_case(ops, a):
     if ((uneven_lengths(seq_rows) and planned_list_pays(len(seq_rows), kvh)) or a.planned) and not a.same_splits:
         # decoded tokens of requests that differ widely in length: splits planned request by request, as the engine does
         entries, most = decode_items(seq_rows, nh, kvh, hd)
-        batch.extras[("attention_decode_items", nh // kvh, tile_columns(hd), kvh)] = (
+        batch.extras[("attention_decode_items", nh // kvh, tile_columns(hd), kvh, 0)] = (
             torch.from_numpy(entries).reshape(-1).to(ops.device), len(entries), most)
     else:
         nb, items, tiles, steps = attention_items(seq_rows, nh // kvh, 0 if a.no_tiles else tile_columns(hd),
                                                   0 if a.tiles else kvh)
         both = torch.from_numpy(np.ascontiguousarray(np.concatenate((items, tiles)))).reshape(-1).to(ops.device)
-        batch.extras[("attention_items", nh // kvh, tile_columns(hd), kvh)] = (both, len(items), nb, len(tiles), steps)
+        batch.extras[("attention_items", nh // kvh, tile_columns(hd), kvh, 0)] = (both, len(items), nb, len(tiles), steps)
     us = graph_time(lambda: ops.paged_attention(q, plane, batch, "g", nh, kvh, hd), a.reps)
     kv_bytes = sum(p0 + n for p0, n in segs) * kvh * hd * 2 * 2
     flops = sum(4 * nh * hd * (n * p0 + n * (n + 1) / 2) for p0, n in segs)
@@ -93,12 +93,21 @@ def attention_case(ops, a):
 def product_case(ops, a):
     m, n, k = a.rows, a.out, a.inner
     x = torch.randn(m, k, device=ops.device).to(torch.bfloat16)
-    w = (torch.randn(n, k, device=ops.device) * k ** -0.5).to(torch.bfloat16)
+    # --copies: the launches take their weights from that many matrices in turn, so that with enough of them (their
+    # bytes beyond the 256 MB of the memory-side cache) every launch streams its weights from HBM as in a decode step
+    ws = [(torch.randn(n, k, device=ops.device) * k ** -0.5).to(torch.bfloat16) for _ in range(max(1, a.copies))]
     res = torch.randn(m, n, device=ops.device).to(torch.bfloat16)
     rms = (torch.ones(k, device=ops.device), 1e-6)
-    kinds = {"plain": lambda: ops.linear(x, w), "residual": lambda: ops.linear(x, w, residual=res),
-             "norm": lambda: ops.linear(x, w, rms=rms), "norm+gate": lambda: ops.linear_swiglu(x, w, rms=rms),
-             "logits": lambda: ops.linear(x, w, out_dtype=torch.float32)}
+    turn = [0]
+
+    def w():
+        turn[0] += 1
+        return ws[turn[0] % len(ws)]
+    kinds = {"plain": lambda: ops.linear(x, w()), "residual": lambda: ops.linear(x, w(), residual=res),
+             "norm": lambda: ops.linear(x, w(), rms=rms), "norm+gate": lambda: ops.linear_swiglu(x, w(), rms=rms),
+             "logits": lambda: ops.linear(x, w(), out_dtype=torch.float32)}
+    if a.few_rows:
+        ops.few_rows = a.few_rows
     us = graph_time(kinds[a.kind], a.reps)
     print(f"product {a.kind} rows {m} out {n} in {k}: {us:.2f} us; weights {n * k * 2 / 1e6:.1f} MB -> "
           f"{n * k * 2 / us / 1e6:.2f} TB/s; {2 * m * n * k / us / 1e6:.1f} TFLOP/s")
@@ -125,6 +134,8 @@ def main(argv=None) -> int:
     pr.add_argument("--out", type=int, default=8192)
     pr.add_argument("--in", dest="inner", type=int, default=1536)
     pr.add_argument("--kind", choices=["plain", "residual", "norm", "norm+gate", "logits"], default="plain")
+    pr.add_argument("--copies", type=int, default=1, help="weight matrices that the launches take in turn")
+    pr.add_argument("--few-rows", type=int, default=0, help="the row count up to which the few-row kernel is used (0: as built)")
     for p in (at, pr):
         p.add_argument("--reps", type=int, default=20)
         p.add_argument("--device", default="cuda:0")

@@ -66,14 +66,14 @@ class GqaAttention:
     def plan_key(self):
         if not hasattr(self.ops, "plan_attention"):
             return None
-        return ("attention", self.n_heads, self.n_kv_heads, self.head_dim)
+        return ("attention", self.n_heads, self.n_kv_heads, self.head_dim, self.window)
 
     def plan_mode(self, seq_rows):
         mode = getattr(self.ops, "plan_attention_mode", None)
-        return mode(seq_rows) if mode is not None else None
+        return mode(seq_rows, self.window) if mode is not None else None
 
     def plan_rows(self, seq_rows, add, mode=None):
-        return self.ops.plan_attention(self.n_heads, self.n_kv_heads, self.head_dim, seq_rows, add, mode)
+        return self.ops.plan_attention(self.n_heads, self.n_kv_heads, self.head_dim, seq_rows, add, mode, self.window)
 
     def forward(self, x, ctx, residual=None, norm=None):
         ops, b = self.ops, ctx.batch

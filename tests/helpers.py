@@ -264,3 +264,64 @@ def slot_pressure_workload(name: str):
     params = [SamplingParams(max_new_tokens=k, temperature=0.0, ignore_eos=True) for k in new]
     want = [pm.greedy_generate(p, k, w, cfg) for p, k in zip(prompts, new)]
     return folder, prompts, params, want
+
+
+# ---- many sampled requests through the scheduler: more live requests than captured steps have exact shapes for ------
+
+def sampled_workload(name: str, n_req: int, seed: int, temperature: float = 0.3, rep_penalty: float = 1.3):
+    """`n_req` requests of mixed prompt and output lengths, sampled with a temperature and a repetition penalty, each
+    from its own random stream: (prompts, sampling params)."""
+    from tiny_inference_server_amd.sampling import SamplingParams
+    rng = random.Random(seed)
+    vocab = TINY[name]["cfg"].vocab_size
+    prompts = [random_ids(vocab, rng.randint(18, 60), seed + 1 + i) for i in range(n_req)]
+    params = [SamplingParams(max_new_tokens=rng.randint(10, 22), temperature=temperature, rep_penalty=rep_penalty,
+                             seed=seed + i, ignore_eos=True) for i in range(n_req)]
+    return prompts, params
+
+
+def fill_cache_with_nan(engine) -> None:
+    """Whatever a kernel reads of a page that its row may not see is then not a number."""
+    for g in engine.cache.groups.values():
+        g.storage.fill_(float("nan"))
+
+
+def watch_decode_steps(engine):
+    """Records, for every step of single tokens that goes through the captured-step path, (requests in the step,
+    whether it was replayed from a kept step). Returns the list that fills up."""
+    seen = []
+    inner = engine._decode_step
+
+    def watching(batch_entries):
+        before = engine.graph_replays
+        out = inner(batch_entries)
+        seen.append((len(batch_entries), engine.graph_replays > before))
+        return out
+    engine._decode_step = watching
+    return seen
+
+
+def check_sampled_tokens(folder, prompts, params, outs, slack: float):
+    """Every generated token against the reference's sampling rule (server.py:22-50) on the plain model's logits for
+    the tokens before it, with the request's own uniform number u. The draw inverts the cumulative distribution in
+    token order and is monotone in u, so a token must lie between the plain draws at u - slack and u + slack: `slack`
+    is what the compute dtype's rounding may move the cumulative mass by (1e-5 in 32-bit). Returns (tokens checked,
+    tokens equal to the plain draw at u itself)."""
+    from tiny_inference_server_amd.sampling import uniform_for
+    cfg, w = pm.read_model_folder(folder)
+    checked = equal = 0
+    for prompt, sp, out in zip(prompts, params, outs):
+        assert len(out) == sp.max_new_tokens
+        ids = list(prompt) + list(out)
+        logits = pm.logits_of(pm.trunk_hidden(ids[:-1], w, cfg), w, cfg)
+        for i, tok in enumerate(out):
+            p = len(prompt) - 1 + i
+            probs = pm.sampling_probs(logits[p], sp.temperature, sp.top_k, sp.top_p, sp.rep_penalty, ids[:p + 1])
+            u = uniform_for(sp.seed, i)
+            lo = pm.pick_by_uniform(probs, max(0.0, u - slack))
+            hi = pm.pick_by_uniform(probs, u + slack) if u + slack < 1.0 else int(torch.nonzero(probs)[-1])
+            assert lo <= tok <= hi, (prompt[:3], i, tok, lo, hi)
+            assert probs[tok] > 0
+            checked += 1
+            equal += tok == pm.pick_by_uniform(probs, u)
+    return checked, equal

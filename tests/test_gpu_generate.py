@@ -79,6 +79,36 @@ def test_bfloat16_scheduler_with_heads_and_preemption():
     assert s.engine.free_pages() == s.engine.total_pages()
 
 
+def test_scheduler_at_the_headline_geometry_with_fourteen_sampled_requests_on_a_pool_of_nan():
+    """Where the captured steps' filler lines, per-request attention splits, preemption, the prediction heads and the
+    sampling kernel's penalty tables meet: 14 requests at the headline model's layer sizes (12 query heads of 128 over
+    3, width 1536) in bfloat16, heads run at every step, plan "cur" on a pool that cannot hold them all, sampled with a
+    temperature and a repetition penalty, every page filled with NaN beforehand (reference's model-level check of its
+    scheduler: test_server.py:66-118). Steps of 9 to 14 decoded tokens are filled up to 16 lines with the cache
+    manager's own request and replayed from captured graphs; every token lies where the reference's sampling rule
+    puts it on the plain model's logits, up to what bfloat16 moves the cumulative distribution by."""
+    from tiny_inference_server_amd.engine import Engine
+    from tiny_inference_server_amd.engine.scheduler import Request, Scheduler
+    name, n_req = "E", 14
+    folder = H.model_folder(name, "bfloat16")
+    prompts, params = H.sampled_workload(name, n_req, seed=300)
+    eng = Engine(folder, dtype="bfloat16", page_size=16, max_tokens=47 * 16, max_requests=n_req, run_heads=True)
+    H.fill_cache_with_nan(eng)
+    steps = H.watch_decode_steps(eng)
+    s = Scheduler(eng, max_batch=n_req, token_budget=96, plan="cur")
+    reqs = [Request(p, sp) for p, sp in zip(prompts, params)]
+    for r in reqs:
+        s.submit(r)
+    s.run()
+    assert s.preempts > 0 and s.replays > 0 and eng.graph_replays > 0
+    assert any(n > 8 and n % 8 and replayed for n, replayed in steps), steps       # a filled-up shape was replayed
+    assert s.peak_running > 8
+    checked, equal = H.check_sampled_tokens(folder, prompts, params, [r.out_ids() for r in reqs], slack=0.08)
+    assert checked == sum(sp.max_new_tokens for sp in params) and equal >= checked // 3, (checked, equal)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages() and eng.cache.n_live == 0
+
+
 def test_temperature_sampling_with_seeded_streams():
     """Tiny B's workload: temperature 0.8, seed 0, mixed chunked prefill and decode; token by token the draw is the
     plain rule's (server.py:22-50) on the plain logits with the request's own uniform number."""

@@ -487,6 +487,44 @@ def test_sampling(sampling_kernel, V):
     assert ops.argmax(logits.cuda()).cpu().tolist() == logits.argmax(-1).tolist()
 
 
+@pytest.mark.parametrize("V", [1000, 48000])
+def test_sampling_against_the_reference_rule(sampling_kernel, V):
+    """The kernel's draws against the reference's rule itself, as the plain implementation states it from
+    server.py:22-50 (sort, top-k cut, cumulative top-p cut that keeps the first token across p, softmax), and not
+    against a restatement of the kernel's method: 16 rows of mixed temperature, top-k, top-p and repetition penalty,
+    7 uniform numbers each. A draw within 2e-6 of a token's edge in the cumulative distribution may be either
+    neighbour (the kernel sums in 32-bit)."""
+    import plain_model as pm
+    ops = sampling_kernel
+    n = 16
+    logits = rnd((n, V), torch.float32, 260, 3.0)
+    rng = random.Random(261)
+    temperature = [rng.choice((0.5, 0.8, 0.9, 1.0, 1.3)) for _ in range(n)]
+    top_k = [rng.choice((0, 0, 2, 5, 50, 200)) for _ in range(n)]
+    top_p = [rng.choice((0.0, 0.0, 0.3, 0.9, 0.95)) for _ in range(n)]
+    pen = [rng.choice((1.0, 1.0, 1.1, 1.3, 2.0)) for _ in range(n)]
+    top_k[0], top_p[0], pen[0] = 50, 0.95, 1.1                      # the reference's run defaults (server.py:515-516)
+    temperature[0] = 0.9
+    # contexts that hold the rows' likeliest tokens, so that the penalty moves the draw
+    ctx = [sorted(set(torch.topk(logits[i], 6).indices.tolist() + rng.choices(range(V), k=9))) for i in range(n)]
+    off = torch.tensor([0] + list(torch.tensor([len(c) for c in ctx]).cumsum(0)), dtype=torch.int32)
+    ctx_t = torch.tensor([t for c in ctx for t in c], dtype=torch.int32)
+    probs = [pm.sampling_probs(logits[i], temperature[i], top_k[i], top_p[i], pen[i], ctx[i]) for i in range(n)]
+    as_t = lambda v, dt: torch.tensor(v, dtype=dt).cuda()
+    strict = 0
+    for trial in range(7):
+        u = torch.rand(n, generator=torch.Generator().manual_seed(270 + trial))
+        got = ops.sample(logits.cuda(), as_t(temperature, torch.float32), as_t(top_k, torch.int32), as_t(top_p, torch.float32),
+                         as_t(pen, torch.float32), u.cuda(), ctx_t.cuda(), off.cuda()).cpu().tolist()
+        for i in range(n):
+            want = pm.pick_by_uniform(probs[i], float(u[i]))
+            lo, hi = pm.pick_by_uniform(probs[i], max(0.0, float(u[i]) - 2e-6)), pm.pick_by_uniform(probs[i], min(1.0, float(u[i]) + 2e-6))
+            assert got[i] == want or lo <= got[i] <= hi, (trial, i, got[i], want, temperature[i], top_k[i], top_p[i], pen[i])
+            strict += lo == hi
+            assert probs[i][got[i]] > 0
+    assert strict >= 100
+
+
 @pytest.mark.parametrize("V", [300, 48000])
 def test_sampling_with_many_values_at_the_cut(sampling_kernel, V):
     """All logits equal: every value ties at any top-k cut, so all are kept and the draw is uniform over the

@@ -114,90 +114,9 @@ def test_attention_mixer_and_block(name, dtype, tol, n_heads, n_kv, hd):
     assert (got - o).abs().max() <= tol * max(1.0, o.abs().max())
 
 
-# ---- a toy mixer with state of its own, and a toy architecture around it, all defined here -------------------------
+# ---- a toy mixer with state of its own, and a toy architecture around it: defined in tests/toy_parts.py ------------
 
-@MIXERS.register("toy_decay", replace=True)
-class ToyDecayMixer:
-    """s <- decay * s + x for every row in order; y = s . W (+ residual). Its state is one vector per request."""
-
-    @classmethod
-    def tensor_shapes(cls, params):
-        return {"w": (params["d_model"], params["d_model"])}
-
-    @classmethod
-    def cache_need(cls, params):
-        return StateNeed((params["d_model"],), "float32")
-
-    def __init__(self, spec, tensors, ops):
-        self.ops, self.decay = ops, float(spec.params["decay"])
-        self.w = to_compute(ops, tensors.of(spec, "w").t())
-
-    # a portion's rows are walked on the host; when every request brings one token the state is updated with the step's
-    # device arrays alone, and such steps may be captured as graphs
-    graph_safe = "single_rows"
-
-    def forward(self, x, ctx, residual=None):
-        b = ctx.batch
-        if b.max_seq_rows == 1 and b.n_rows == b.n_seqs:
-            slots = b.seq_slots.long()
-            s = self.decay * ctx.state[slots] + x.float()
-            ctx.state[slots] = s
-            return self.ops.linear(s.to(x.dtype), self.w, residual=residual)
-        s_all = torch.empty(x.shape[0], x.shape[1], dtype=torch.float32, device=x.device)
-        for (first, p0, n), slot in zip(ctx.batch.seq_rows, ctx.batch.host_slots):
-            s = ctx.state[slot]
-            for r in range(first, first + n):
-                s = self.decay * s + x[r].float()
-                s_all[r] = s
-            if n:
-                ctx.state[slot] = s
-        return self.ops.linear(s_all.to(x.dtype), self.w, residual=residual)
-
-
-@dataclass(frozen=True)
-class ToyConfig:
-    d_model: int
-    vocab_size: int
-    hidden: int
-    decay: float
-    max_context: int = 128
-    architecture: str = "ToyStateModel"
-
-    @classmethod
-    def from_dict(cls, raw):
-        return cls(raw["d_model"], raw["vocab_size"], raw["hidden"], raw["decay"], raw.get("max_context", 128))
-
-    def to_dict(self):
-        return dict(self.__dict__)
-
-
-def toy_spec(cfg):
-    norm = lambda n: PartSpec("norm", "rmsnorm_l2", {"width": cfg.d_model, "eps": 1e-6}, {"gain": n})
-    layers = []
-    for l in range(2):
-        mixer = PartSpec("mixer", "toy_decay", {"d_model": cfg.d_model, "decay": cfg.decay}, {"w": f"l{l}.mix.w"})
-        ffn = PartSpec("feed_forward", "swiglu", {"d_model": cfg.d_model, "hidden": cfg.hidden},
-                       {"gate": f"l{l}.g", "up": f"l{l}.u", "down": f"l{l}.d"})
-        layers.append(LayerSpec("prenorm_residual", {"mixer": mixer, "mixer_norm": norm(f"l{l}.n1"),
-                                                     "feed_forward": ffn, "feed_forward_norm": norm(f"l{l}.n2")}))
-    # the run order is data: layer 0, layer 1, then layer 0 again with a state of its own
-    stage = StageSpec("trunk", 0, PartSpec("stage_input", "token_embedding"),
-                      (LayerCall(0), LayerCall(1), LayerCall(0)), norm("out"))
-    return ModelSpec(cfg.d_model, cfg.vocab_size, cfg.max_context, tuple(layers), (stage,), "emb", "emb")
-
-
-def toy_plain(ids, w, cfg):
-    x = w["emb"][torch.tensor(ids)].double()
-    for l in (0, 1, 0):
-        a = pm.rms_norm(x, w[f"l{l}.n1"].double(), 1e-6)
-        s, rows = torch.zeros(cfg.d_model, dtype=torch.float64), []
-        for r in range(len(ids)):
-            s = cfg.decay * s + a[r]
-            rows.append(s)
-        x = x + torch.stack(rows) @ w[f"l{l}.mix.w"].double()
-        x = x + pm.swiglu_ffn(pm.rms_norm(x, w[f"l{l}.n2"].double(), 1e-6), w[f"l{l}.g"].double(), w[f"l{l}.u"].double(),
-                              w[f"l{l}.d"].double())
-    return pm.rms_norm(x, w["out"].double(), 1e-6) @ w["emb"].double().T
+from toy_parts import ToyConfig, ToyDecayMixer, toy_plain, toy_spec
 
 
 def test_toy_mixer_with_state_is_registered_built_and_stepped():
@@ -226,6 +145,39 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
         assert (lg.double() - want).abs().max() <= 2e-5 * max(1.0, want.abs().max()), (rid, p)
     ARCHITECTURES.unregister("ToyStateModel")
     MIXERS.unregister("toy_decay")
+
+
+def test_command_line_and_generate_take_a_toy_architecture(tmp_path, capsys):
+    """The command line and generate() with a model folder of an architecture registered from here, whose
+    configuration class is not the built-in one and whose mixers keep no pages: the pool's size in bytes is turned
+    into pages by what the parts keep (nothing), the prompts are drawn from the spec's vocabulary, and the tokens
+    are the plain toy model's."""
+    from tiny_inference_server_amd.__main__ import main
+    from tiny_inference_server_amd.engine.generate import generate
+    from tiny_inference_server_amd.weights import write_random_model
+    ARCHITECTURES.register("ToyStateModel", Architecture("ToyStateModel", ToyConfig, toy_spec), replace=True)
+    MIXERS.register("toy_decay", ToyDecayMixer, replace=True)
+    try:
+        cfg = ToyConfig(d_model=48, vocab_size=101, hidden=80, decay=0.7)
+        folder = write_random_model(cfg, 9, str(tmp_path / "toy"), std=0.1, gain_jitter=0.1, dtype="float32")
+        w = random_tensors(cfg, 9, std=0.1, gain_jitter=0.1, dtype="float32")
+
+        def greedy(prompt, n):
+            ids = list(prompt)
+            for _ in range(n):
+                ids.append(int(torch.argmax(toy_plain(ids, w, cfg)[-1])))
+            return ids[len(prompt):]
+        prompts = [H.random_ids(101, n, 60 + i) for i, n in enumerate((11, 3, 17))]
+        assert generate(folder, prompts, max_new_tokens=5, temperature=0.0, dtype="float32", max_batch=2,
+                        token_budget=8) == [greedy(p, 5) for p in prompts]
+        capsys.readouterr()
+        assert main(["--model", folder, "--dtype", "float32", "--prompt-ids", "5,17,3", "--prompt-ids", "9",
+                     "--max-new-tokens", "4", "--greedy", "--pool-bytes", "1MiB", "--max-batch", "2"]) == 0
+        lines = [l.split()[1:] for l in capsys.readouterr().out.splitlines() if l.startswith("OUTPUT:")]
+        assert [[int(t) for t in l] for l in lines] == [greedy([5, 17, 3], 4), greedy([9], 4)]
+    finally:
+        ARCHITECTURES.unregister("ToyStateModel")
+        MIXERS.unregister("toy_decay")
 
 
 # ---- toy arrangements: a block with no feed-forward, and a block with two mixers, each with a cache of its own ------

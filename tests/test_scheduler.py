@@ -195,3 +195,28 @@ def test_static_admission_waits_for_pages_instead_of_preempting(greedy_truth):
                       return_scheduler=True)
     assert out == greedy_truth and s.preempts == 0 and s.peak_running <= 3
     assert eng.free_pages() == eng.total_pages() == 6
+
+
+def test_twelve_sampled_requests_with_heads_on_a_pool_of_nan_through_kept_steps():
+    """The GPU suite's schedule at the headline geometry, here in 32-bit on the stand-in with kept steps emulated, so
+    that the host side alone is on trial: more live requests than captured steps have exact shapes for (filler lines),
+    the prediction heads run, plan "cur" preempts, sampling with temperature and repetition penalty from per-request
+    streams, pages full of NaN beforehand. Every token is the reference rule's draw on the plain model's logits."""
+    name, n_req = "A", 12
+    folder = H.model_folder(name, "float32")
+    prompts, params = H.sampled_workload(name, n_req, seed=310, temperature=0.7, rep_penalty=1.3)
+    eng = Engine(folder, dtype="float32", page_size=16, max_tokens=40 * 16, max_requests=n_req,
+                 ops=TorchOps(graphs=True), run_heads=True)
+    H.fill_cache_with_nan(eng)
+    steps = H.watch_decode_steps(eng)
+    s = Scheduler(eng, max_batch=n_req, token_budget=64, plan="cur")
+    reqs = [Request(p, sp) for p, sp in zip(prompts, params)]
+    for r in reqs:
+        s.submit(r)
+    s.run()
+    assert s.preempts > 0 and s.replays > 0
+    assert any(n > 8 and n % 8 and replayed for n, replayed in steps), steps
+    checked, equal = H.check_sampled_tokens(folder, prompts, params, [r.out_ids() for r in reqs], slack=1e-5)
+    assert checked == sum(sp.max_new_tokens for sp in params) and equal >= checked - 2, (checked, equal)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages() and eng.cache.n_live == 0

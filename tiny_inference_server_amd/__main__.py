@@ -71,7 +71,7 @@ def main(argv=None) -> int:
                     help="also run the multi-token-prediction heads at every step (their drafts are not used)")
     a = ap.parse_args(argv)
 
-    from .config import load_config
+    from .config import ARCHITECTURES, load_config
     from .engine import Engine
     from .engine.generate import generate
     from .weights import write_random_model
@@ -92,15 +92,14 @@ def main(argv=None) -> int:
         prompts = [[int(t) for t in p.replace(" ", "").split(",") if t] for p in a.prompt_ids]
     else:
         rng = random.Random(a.seed)
-        prompts = [[rng.randrange(cfg.vocab_size) for _ in range(a.prompt_len)] for _ in range(a.num_prompts)]
+        vocab = ARCHITECTURES.get(cfg.architecture).build_spec(cfg).vocab_size
+        prompts = [[rng.randrange(vocab) for _ in range(a.prompt_len)] for _ in range(a.num_prompts)]
 
-    elem = 2 if a.dtype == "bfloat16" else 4
-    planes = cfg.n_layers + (cfg.mtp_heads if a.heads else 0)
-    page_bytes = a.tokens_per_block * 2 * cfg.n_kv_heads * cfg.head_dim * planes * elem      # block_table.py:34-38
-    n_pages = max(1, parse_bytes(a.pool_bytes) // page_bytes)
-    engine = Engine(model_dir, dtype=a.dtype, page_size=a.tokens_per_block, n_pages=n_pages,
+    # as many pages as the bytes hold, whatever the model's parts keep in a page (reference block_table.py:34-38)
+    engine = Engine(model_dir, dtype=a.dtype, page_size=a.tokens_per_block, pool_bytes=parse_bytes(a.pool_bytes),
                     max_requests=a.max_batch, device=a.device, run_heads=a.heads)
-    print(f"POOL: {n_pages} blocks of {a.tokens_per_block} tokens", file=sys.stderr)
+    if engine.cache.groups:
+        print(f"POOL: {engine.total_pages()} blocks of {a.tokens_per_block} tokens", file=sys.stderr)
     import torch
     t0 = time.time()
     outs, sched = generate(engine, prompts, max_new_tokens=a.max_new_tokens,

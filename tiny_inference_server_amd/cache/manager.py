@@ -262,6 +262,32 @@ class CacheManager:
             if g.spec.window > 0:
                 g.release_behind(slot, next_position - max_lag - g.spec.window + 1)
 
+    def pages_to_hold(self, n_positions: int, step_positions: int = 0, max_lag: int = 0) -> Dict[str, int]:
+        """Pages of each group that a request holds at the most while it grows to `n_positions`, fed at most
+        `step_positions` a step: every page of its positions, or, in a window group, the pages of a window, of the
+        stages' lag and of one step's positions (what is released behind a step is released after it)."""
+        out = {}
+        for name, g in self.groups.items():
+            pages = -(-n_positions // self.page_size)
+            if g.spec.window > 0:
+                span = g.spec.window + max_lag + max(1, step_positions or n_positions)
+                pages = min(pages, -(-span // self.page_size) + 1)
+            out[name] = pages
+        return out
+
+    @staticmethod
+    def page_bytes(needs: Mapping[str, object], page_size: int, dtype) -> int:
+        """Bytes that one more page costs: every group gets as many pages as every other, and a page of a group has
+        a plane for each of the group's cache users (the reference's one geometry: block_table.py:34-38)."""
+        elem = torch.empty(0, dtype=dtype).element_size()
+        return sum(2 * need.n_kv_heads * need.head_dim * page_size * elem
+                   for need in needs.values() if isinstance(need, PagedKvNeed))
+
+    def bytes_per_position(self) -> int:
+        """Bytes of keys and values that one position of one request takes, over all groups and planes."""
+        elem = torch.empty(0, dtype=self.dtype).element_size()
+        return sum(len(g.spec.keys) * 2 * g.spec.n_kv_heads * g.spec.head_dim * elem for g in self.groups.values())
+
     def free_pages(self) -> Dict[str, int]:
         return {name: g.pool.n_free for name, g in self.groups.items()}
 

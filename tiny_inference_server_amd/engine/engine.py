@@ -48,8 +48,10 @@ class StepOutput:
 class Engine:
     def __init__(self, model_dir: Optional[str] = None, *, config=None, tensors=None, dtype="bfloat16",
                  page_size: int = 16, max_tokens: Optional[int] = None, n_pages: Optional[int] = None,
-                 max_requests: int = 64, device="cuda:0", ops=None, use_graphs: bool = True,
-                 run_heads: bool = True):
+                 pool_bytes: Optional[int] = None, max_requests: int = 64, device="cuda:0", ops=None,
+                 use_graphs: bool = True, run_heads: bool = True):
+        """The cache's size is given as tokens (`max_tokens`), pages (`n_pages`) or bytes (`pool_bytes`: as many
+        pages as fit, whatever groups and planes the model's parts ask for)."""
         self.dtype = resolve_dtype(dtype)
         if model_dir is not None:
             config = load_config(model_dir)
@@ -71,9 +73,14 @@ class Engine:
         # prediction heads' weights are still loaded and checked, but they take no time and no cache
         self.run_spec = self.spec if run_heads else dataclasses.replace(self.spec, stages=self.spec.stages[:1])
         self.model = Model(self.run_spec, tensors, ops)
+        if n_pages is None and pool_bytes is not None:
+            per_page = CacheManager.page_bytes(self.model.cache_needs(), page_size, self.dtype)
+            n_pages = max(1, int(pool_bytes) // per_page) if per_page else 1
         if n_pages is None:
             if max_tokens is None:
-                raise ValueError("give the cache's size as max_tokens or n_pages")
+                if CacheManager.page_bytes(self.model.cache_needs(), page_size, self.dtype):
+                    raise ValueError("give the cache's size as max_tokens, n_pages or pool_bytes")
+                max_tokens = page_size          # no part keeps pages: the size is of no consequence
             n_pages = -(-int(max_tokens) // page_size)
         self.page_size = page_size
         # decode steps are replayed from captured graphs where the kernels allow it
@@ -143,16 +150,26 @@ class Engine:
     def fed(self, rid: Hashable) -> int:
         return self.requests[rid][1]
 
+    # Pages, as one number for whoever plans above the step function: every group has as many pages as every other,
+    # so what binds is the group that needs the most. A model without paged groups (its mixers keep state of fixed
+    # size only) needs none and never runs out.
+    NO_PAGE_LIMIT = 1 << 40
+
     def pages_to_grow(self, rid: Hashable, n_tokens: int) -> int:
         """Most pages any group must take so that `rid` can be fed `n_tokens` more."""
         slot, fed = self.requests[rid]
         return max(self.cache.pages_needed(slot, fed + n_tokens).values(), default=0)
 
+    def pages_to_hold(self, n_positions: int, step_positions: int = 0) -> int:
+        """Most pages any group holds at a time for a request that grows to `n_positions`, fed at most
+        `step_positions` a step (a window group gives pages back as it goes)."""
+        return max(self.cache.pages_to_hold(n_positions, step_positions, self.model.max_lag).values(), default=0)
+
     def free_pages(self) -> int:
-        return min(self.cache.free_pages().values(), default=0)
+        return min(self.cache.free_pages().values(), default=self.NO_PAGE_LIMIT)
 
     def total_pages(self) -> int:
-        return min(self.cache.total_pages().values(), default=0)
+        return min(self.cache.total_pages().values(), default=self.NO_PAGE_LIMIT)
 
     # ---- the step ------------------------------------------------------------------------------------
     @torch.no_grad()

@@ -160,8 +160,9 @@ class Model:
         """Logits of every stage at the n wanted places from one product with the output table, which all stages
         share (reference main_models_new.py:225-226): the table is read once however many stages there are.
         Returns (first stage's logits [n, vocab], [logits of each further stage], [which of their rows are valid]);
-        rows that a later stage does not have yet come back as NaN. The first stage's part equals `logits` bit for
-        bit: same gather, same product, a row's result does not depend on the other rows."""
+        rows that a later stage does not have yet come back as NaN. The first stage's part is what `logits` gives: the
+        same gather and the same product on the same rows (up to the order of 32-bit partial sums, which the product
+        may choose by the number of rows)."""
         vocab, S = self.spec.vocab_size, len(outs)
         if n == 0:
             e = torch.empty(0, vocab, dtype=torch.float32, device=self.ops.device)

@@ -103,13 +103,18 @@ class Scheduler:
             raise ValueError(f"a prompt of {req.prompt_len} tokens leaves no room in a context of {self.max_context}")
         self.queue.append(req)
 
-    def _held(self, r: Request) -> int:
-        tokens = max(r.fed, r.reserved)
-        return pages_for(tokens, self.page_size) if tokens else 0
-
+    # How many pages something takes is the engine's knowledge (its cache manager's groups: all keys, a window of
+    # them, none at all); the scheduler only adds, compares and decides.
     def _grow_pages(self, r: Request, n_new: int) -> int:
-        """Pages r must take to be fed n_new more tokens."""
-        return max(0, pages_for(r.fed + n_new, self.page_size) - self._held(r))
+        """Pages r must take to be fed n_new more tokens (a request is known to the engine from its first step, or
+        from a static reservation, on)."""
+        if r.id in self.engine.requests:
+            return self.engine.pages_to_grow(r.id, n_new)
+        return self.engine.pages_to_hold(r.fed + n_new, n_new)
+
+    def _pages_for(self, n_tokens: int) -> int:
+        """Pages a request of n_tokens holds at the most, fed under this scheduler's token budget."""
+        return self.engine.pages_to_hold(n_tokens, self.token_budget)
 
     def _reserve_tokens(self, r: Request) -> int:
         """Tokens a static mode reserves at admission (reference server.py:180-185)."""
@@ -121,7 +126,7 @@ class Scheduler:
 
     def _final_pages(self, r: Request) -> int:
         """Pages r holds once it has generated all it may (the last token is sampled, never fed)."""
-        return pages_for(min(r.prompt_len + r.params.max_new_tokens - 1, self.max_context), self.page_size)
+        return self._pages_for(min(r.prompt_len + r.params.max_new_tokens - 1, self.max_context))
 
     def admit(self) -> None:
         total = self.engine.total_pages()
@@ -130,7 +135,9 @@ class Scheduler:
         budget = self.engine.free_pages() - sum(self._grow_pages(r, len(r.ids) - r.fed) for r in self.active)
         while self.queue and len(self.active) < self.max_batch:
             q = self.queue[0]
-            need_now = pages_for(max(len(q.ids), self._reserve_tokens(q)) if self.static else len(q.ids), self.page_size)
+            tokens_now = max(len(q.ids), self._reserve_tokens(q)) if self.static else len(q.ids)
+            # (a reservation takes every position's page, also where a window would give pages back)
+            need_now = self.engine.pages_to_hold(tokens_now, tokens_now) if self.static else self._pages_for(tokens_now)
             if self.static and need_now > total:
                 raise RuntimeError(f"static reservation {need_now} pages > pool {total}")
             if self.plan == "final" and not self.static:
@@ -191,7 +198,7 @@ class Scheduler:
             if len(self.active) == 1:
                 r = self.active[0]
                 raise RuntimeError("kv pool too small for a single request: "
-                                   f"{len(r.ids)} tokens need {pages_for(len(r.ids), self.page_size)} pages of "
+                                   f"{len(r.ids)} tokens need {self._pages_for(len(r.ids))} pages of "
                                    f"{self.page_size}, the pool has {self.engine.total_pages()}")
             self.preempt()
         self.peak_running = max(self.peak_running, len(self.active))

@@ -63,8 +63,12 @@ class FusePreviousStage:
             return ops.empty(0, D)
         fused = ops.empty(batch.n_rows, 2 * D)
         ops.gather_rows(previous if previous is not None else state, state, batch.source_index, out=fused[:, :D])
-        ops.embedding_rmsnorm(shared["embedding"], batch.tokens, self.embed_norm.gain, self.embed_norm.eps,
-                              out=fused[:, D:])
+        if hasattr(self.embed_norm, "as_rms"):
+            # a norm that offers its (gain, eps) is fused into the gather
+            gain, eps = self.embed_norm.as_rms()
+            ops.embedding_rmsnorm(shared["embedding"], batch.tokens, gain, eps, out=fused[:, D:])
+        else:
+            fused[:, D:].copy_(self.embed_norm(ops.embedding(shared["embedding"], batch.tokens)))
         return ops.linear(fused, self.w_proj)
 
     def after_step(self, batch, previous, state):

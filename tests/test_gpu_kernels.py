@@ -592,7 +592,7 @@ def test_library_product_at_listed_widths(ops_for):
     ops = ops_for(torch.bfloat16)
     for i, (N, K) in enumerate(sorted(ops.library_widths)):
         w = rnd((N, K), torch.bfloat16, 300 + i, K ** -0.5).cuda()
-        for M in (65, 200, 1024, 2047, 2112) + ((4096,) if i % 4 == 0 else ()):
+        for M in (129, 200, 1024, 2047, 2112) + ((4096,) if i % 4 == 0 else ()):
             x, res = rnd((M, K), torch.bfloat16, 400 + i).cuda(), rnd((M, N), torch.bfloat16, 500 + i).cuda()
             print(f"library product: rows {M} (asked {library_rows(M)}), out {N}, in {K}", flush=True)
             got = ops.linear(x, w, residual=res)

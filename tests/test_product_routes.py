@@ -25,7 +25,7 @@ class Recorder:
         return call
 
 
-def host_ops(widths=None, few_rows=64):
+def host_ops(widths=None, few_rows=hip_ops._FEW_ROWS):
     """The operations object without a device: its dispatch is real, its libraries record."""
     ops = object.__new__(HipOps)
     ops.device = torch.device("cpu")
@@ -60,8 +60,10 @@ def test_library_rows_family():
 def test_routes():
     w = {(2304, 1536)}
     assert product_route(8, 2304, 1536, True, False, w) == "few_rows"
-    assert product_route(64, 2304, 1536, True, False, w) == "few_rows"
-    assert product_route(65, 2304, 1536, True, False, w) == "library"
+    assert product_route(64, 2304, 1536, True, False, w, few_rows=64) == "few_rows"
+    assert product_route(65, 2304, 1536, True, False, w, few_rows=64) == "library"
+    assert product_route(hip_ops._FEW_ROWS, 2304, 1536, True, False, w) == "few_rows"
+    assert product_route(hip_ops._FEW_ROWS + 1, 2304, 1536, True, False, w) == "library"
     assert product_route(2048, 2304, 1536, True, True, w) == "few_rows"         # 32-bit results: own kernels
     assert product_route(2048, 6144, 4096, True, False, w) == "few_rows"        # a width nobody listed
     assert product_route(2048, 2304, 1536, False, False, w) == "plain"
@@ -121,24 +123,24 @@ def test_rows_beyond_a_callers_tensor_are_never_read():
     """A tensor from outside has no memory behind its last row: the product runs on a copy that has."""
     ops = host_ops()
     N, K = sorted(library_widths())[0]
-    M = 100
+    M = 170
     x = torch.empty(M, K, dtype=torch.bfloat16)
     res = torch.empty(M, N, dtype=torch.bfloat16)
     ops.linear(x, torch.empty(N, K, dtype=torch.bfloat16), residual=res)
     fn, a = [c for c in ops.calls if c[0] == "tis_gemm_library"][0]
-    assert a[7] == 128
+    assert a[7] == 192
     assert a[0] != x.data_ptr() and a[3] != res.data_ptr()
     # and one made by the operations object is used where it lies
     ops.calls.clear()
     x2, res2 = ops.empty(M, K), ops.empty(M, N)
     ops.linear(x2, torch.empty(N, K, dtype=torch.bfloat16), residual=res2)
     fn, a = [c for c in ops.calls if c[0] == "tis_gemm_library"][0]
-    assert a[0] == x2.data_ptr() and a[3] == res2.data_ptr() and HipOps._holds_rows(x2, 128)
+    assert a[0] == x2.data_ptr() and a[3] == res2.data_ptr() and HipOps._holds_rows(x2, 192)
 
 
 def test_unaligned_operands_go_to_the_plain_kernel():
     ops = host_ops()
-    x = torch.empty(100, 1544, dtype=torch.bfloat16)[:, 3:1539]      # rows start 6 bytes into a 16-byte piece
+    x = torch.empty(300, 1544, dtype=torch.bfloat16)[:, 3:1539]      # rows start 6 bytes into a 16-byte piece
     ops.linear(x, torch.empty(2304, 1536, dtype=torch.bfloat16))
     assert [c[0] for c in ops.calls if c[0].startswith("tis_gemm")] == ["tis_gemm_plain"]
 
@@ -146,7 +148,7 @@ def test_unaligned_operands_go_to_the_plain_kernel():
 def test_the_library_path_refuses_an_unlisted_width_even_if_asked_directly():
     ops = host_ops()
     with pytest.raises(KernelError, match="not among"):
-        ops._linear_library(ops.empty(128, 4096), torch.empty(6144, 4096, dtype=torch.bfloat16), None)
+        ops._linear_library(ops.empty(256, 4096), torch.empty(6144, 4096, dtype=torch.bfloat16), None)
 
 
 def test_gated_and_projection_products_follow_the_same_routes():

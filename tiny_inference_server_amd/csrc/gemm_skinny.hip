@@ -1,10 +1,11 @@
 // C[M,N] = f(A[M,K]) . W[N,K]^T for few rows: the matrix product of decode steps, where the job is to stream W from
-// HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950). A workgroup takes up to MB * 16 rows; more rows than that are cut
-// into panels of that many, one per blockIdx.y, each an independent product over the same weights (the panels of a
-// column tile run side by side, so the weights come from HBM once and from the caches after that). That is the right
-// kernel for a few panels; for many, every panel streams all of W again, which only a product tiled in both directions
-// avoids: it still gives the right result, slowly.
+// HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950). Two kernels: up to 16 rows, operands straight from memory into
+// registers (below); from 17 rows on, operands staged through LDS, in panels of 32 rows, one per blockIdx.y, each an
+// independent product over the same weights (the panels of a column tile run side by side, so the weights come from
+// HBM once and from the caches after that). That is right for a few panels; for many, every panel streams all of W
+// again, which only a product tiled in both directions avoids: it still gives the right result, slowly.
 //
+// The kernel for up to 16 rows:
 // One workgroup owns 16 rows of W (16 output columns; 8 in the narrow variant below) over the whole of K; its
 // waves take the 32-wide steps of K in turn, so together they read each weight row in contiguous runs. W rows are the A operand straight from
 // global memory (16 bytes per lane), the activations are the B operand straight from L2 (they are a few KB
@@ -52,12 +53,9 @@ struct RopeArgs {
 // of eight steps, or sixteen waves, so that all of a wave's loads are in flight at once, measured the same within
 // noise (the gated product at 64 rows slower: fewer workgroups fit a compute unit).
 //
-// MB: blocks of 16 rows of X that share every weight tile a wave loads: one or two. More rows than 32 are further
-// panels (blockIdx.y): the panels of a column tile run side by side at the time of one (the down product, 12.6 MB:
-// 14.7 us at 32 rows, 14.6 at 64), which leaves this kernel ahead of the library's product with its separate norm,
-// gate and rotary launches up to 64 rows (whole decode steps at 0.9B, context 1,024, tokens a second, panels /
-// library: batch 48 17.9k / 16.4k, 64 21.4k / 20.3k, 96 24.0k / 24.1k, 128 26.7k / 29.7k). What a workgroup's time
-// goes to from 17 rows on is the activations: it reads all of its panel's X from L2 beside 16 rows of W.
+// MB: blocks of 16 rows of X that share every weight tile a wave loads. One is built: with two, a wave fetches its
+// own pieces of twice the activations, 16 bytes a lane from 16 different rows, and that is what its time went to
+// (down product, 12.6 MB: 7.3 us at 8 rows, 10.4 at 16, 14.7 at 32); 17 rows and more go to the staged kernel.
 //
 // CT: column tiles of 16 a workgroup owns. Two where the matrix is so wide that half as many workgroups still fill
 // the chip: a wave then uses the activations it loaded (and normed) for twice as many weights.
@@ -301,13 +299,328 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
   }
 }
 
+// ---- 17 rows and more: operands staged through LDS ----
+//
+// From two blocks of rows on, what a workgroup of the kernel above spends its time on is the activations: every wave
+// fetches its own pieces of X, 16 bytes a lane from 16 different rows, and of W likewise. Here a workgroup of eight waves
+// owns CT * 16 columns and a panel of MB * 16 rows over the whole of K and walks K in chunks of 256: a chunk's
+// weight rows and activation rows (512 bytes each) are copied into LDS by loads that write LDS directly
+// (global_load_lds_dwordx4: no registers; a wave's load is two whole 512-byte runs), NSTAGE - 1 chunks ahead of the
+// products, and wave w takes the w-th 32-wide step of the chunk for all CT * MB tiles, so the waves' partial sums are
+// added at the end as above, in a fixed order. A row's 32 pieces of 16 bytes lie in LDS with their index XORed by
+// the row's number in its tile, so that the 16 rows an operand fetch reads for one piece index fall into 16
+// different bank groups; the copying lane picks the piece that belongs in its slot. With NORM the gains of a chunk
+// are staged the same way (1 KB, by wave 0).
+#pragma clang diagnostic ignored "-Winline-asm"   // M0 in a clobber list: meant
+// One 16-byte piece per lane from global memory straight into LDS: lane i's piece lands at lds_base + 16 * i. In
+// assembly, because the compiler would order every later LDS read behind such a load, whichever buffer it reads; so
+// the compiler does not count these loads either, and whoever reads the pieces waits for them (vmcnt) and for the
+// other waves (barrier).
+__device__ __forceinline__ void copy16_to_lds(const void* src, const void* lds_base) {
+  // (the base is the same on every lane: into a scalar register, whatever the compiler made of it so far)
+  const unsigned base = (unsigned)__builtin_amdgcn_readfirstlane(
+      (int)(unsigned)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+}
+template <int N_LATER>
+__device__ __forceinline__ void wait_all_but() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N_LATER) : "memory");
+}
+
+template <int MB, int CT, bool NORM, int EPI, typename TO, int NSTAGE>
+__global__ __launch_bounds__(512) void gemm_staged_kernel(
+    const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const float* __restrict__ gain, float eps,
+    const bf16* __restrict__ R_in, long r_ld, TO* __restrict__ C, long c_ld, int M, int N, int K, RopeArgs rope) {
+  constexpr int WAVES = 8, KC = 256;
+  constexpr int ROWS = 16 * (CT + MB);            // rows of a stage: the weight tiles' first, then the activations'
+  constexpr int STAGE = ROWS * 512 + (NORM ? 1024 : 0);
+  constexpr int L = CT + MB;                      // loads of a stage that every wave issues (wave 0: one more for the gains)
+  constexpr int RED = WAVES * MB * CT * 1024 + WAVES * MB * 16 * 4;     // the waves' partial sums at the end
+  constexpr int LDS_BYTES = NSTAGE * STAGE > RED ? NSTAGE * STAGE : RED;
+  static_assert(LDS_BYTES <= 160 * 1024, "stages exceed the LDS of a compute unit");
+  static_assert(L * (NSTAGE - 1) + NSTAGE <= 63, "more loads in flight than the counter counts");
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (16 * CT);
+  {
+    const long m0 = (long)blockIdx.y * (MB * 16);
+    X += m0 * x_ld;
+    C += m0 * c_ld;
+    if (EPI == EPI_RESIDUAL) R_in += m0 * r_ld;
+    if (EPI == EPI_ROPE) {
+      rope.positions += m0;
+      if (rope.write_slots) rope.write_slots += m0;
+    }
+    M = min(M - (int)m0, MB * 16);
+  }
+
+  // What this wave copies of every chunk: L pairs of rows; lane l takes slot l & 31 of row 2 * pair + (l >> 5), which
+  // holds the piece (slot ^ row's number in its tile) of the row's 512 bytes. Rows past the matrix read a row inside.
+  const bf16* row_ptr[L];
+  int piece_k[L];
+#pragma unroll
+  for (int i = 0; i < L; ++i) {
+    const int row = 2 * (i * WAVES + wave) + (lane >> 5);
+    piece_k[i] = ((lane & 31) ^ (row & 15)) * 8;
+    if (row < 16 * CT) {
+      const int n = n0 + row;
+      row_ptr[i] = W + (long)(n < N ? n : N - 1) * K;
+    } else {
+      const int m = row - 16 * CT;
+      row_ptr[i] = X + (long)(m < M ? m : 0) * x_ld;
+    }
+  }
+  const int n_chunks = (K + KC - 1) / KC;
+  auto issue = [&](int c) {
+    unsigned char* st = lds + (c % NSTAGE) * STAGE;
+    const int k0 = c * KC;
+#pragma unroll
+    for (int i = 0; i < L; ++i) {
+      const int k = k0 + piece_k[i];
+      copy16_to_lds(row_ptr[i] + (k < K ? k : 0), st + (i * WAVES + wave) * 1024);
+    }
+    if (NORM && wave == 0) {
+      const int k = k0 + lane * 4;
+      copy16_to_lds(gain + (k < K ? k : 0), st + ROWS * 512);
+    }
+  };
+
+  // What the epilogue wants from memory, asked for before the main loop by the lanes that will use it. Tile t of the
+  // MB x CT tiles is finished by wave t % 8; a result lane (g, c16) holds columns n_out .. n_out + 3 of row m_out.
+  constexpr int TILES = MB * CT, TPW = (TILES + WAVES - 1) / WAVES;
+  float res[TPW][4];
+  float2 cs[TPW][2];
+  int slot[TPW];
+#pragma unroll
+  for (int j = 0; j < TPW; ++j) {
+    const int t = j * WAVES + wave, mb = t / CT, ct = t % CT;
+    const int m = mb * 16 + c16, n_out = n0 + ct * 16 + g * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) res[j][i] = 0.f;
+    cs[j][0] = cs[j][1] = make_float2(1.f, 0.f);
+    slot[j] = 0;
+    if (t >= TILES || m >= M) continue;
+    if (EPI == EPI_RESIDUAL) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n_out + i < N) res[j][i] = static_cast<float>(R_in[(long)m * r_ld + n_out + i]);
+    }
+    if (EPI == EPI_ROPE && n_out < N) {
+      const int hd = rope.head_dim;
+      const int head = n_out / hd, e0 = n_out % hd;
+      if (head < rope.n_heads + rope.n_kv_heads && rope.table) {
+        const long at = (long)rope.positions[m] * (hd / 2) + e0 / 2;
+        cs[j][0] = rope.table[at];
+        cs[j][1] = rope.table[at + 1];
+      }
+      if (head >= rope.n_heads && rope.write_cache) slot[j] = rope.write_slots[m];
+    }
+  }
+
+  f32x4 acc[MB][CT];
+  float ss[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    ss[mb] = 0.f;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc[mb][ct] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+#pragma unroll
+  for (int c = 0; c < NSTAGE - 1; ++c)
+    if (c < n_chunks) issue(c);
+  const int piece = ((wave * 4 + g) ^ c16) * 16;      // where this lane's 16 bytes of a row lie in a stage
+  for (int c = 0; c < n_chunks; ++c) {
+    // this wave's copies of chunk c have landed: all but those of the chunks issued after it may be outstanding
+    // (wave 0 has issued one more per chunk, so it waits a little longer than it must)
+    const int later = min(n_chunks - 1 - c, NSTAGE - 2);
+    if (later <= 0) wait_all_but<0>();
+    else if (later == 1) wait_all_but<L>();
+    else if (later == 2) wait_all_but<2 * L>();
+    else wait_all_but<(NSTAGE - 2) * L>();
+    // ... and everybody's: and every wave is done with chunk c - 1, whose stage the next copies overwrite
+    __builtin_amdgcn_s_barrier();
+    if (c + NSTAGE - 1 < n_chunks) issue(c + NSTAGE - 1);
+    const unsigned char* st = lds + (c % NSTAGE) * STAGE;
+    const bool k_ok = c * KC + wave * 32 + g * 8 < K;     // K is a multiple of 8: a lane's 8 values are all in or all out
+    bf16x8 a[CT], b[MB];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) a[ct] = *reinterpret_cast<const bf16x8*>(st + (ct * 16 + c16) * 512 + piece);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) b[mb] = *reinterpret_cast<const bf16x8*>(st + ((CT + mb) * 16 + c16) * 512 + piece);
+    float gv[8];
+    if (NORM) {
+      const float4 g0 = *reinterpret_cast<const float4*>(st + ROWS * 512 + wave * 128 + g * 32);
+      const float4 g1 = *reinterpret_cast<const float4*>(st + ROWS * 512 + wave * 128 + g * 32 + 16);
+      gv[0] = g0.x; gv[1] = g0.y; gv[2] = g0.z; gv[3] = g0.w;
+      gv[4] = g1.x; gv[5] = g1.y; gv[6] = g1.z; gv[7] = g1.w;
+    }
+    if (!k_ok) {       // past the end of K (the last chunk): whatever was copied there counts as zero
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) a[ct] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) b[mb] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) gv[e] = 0.f;
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      bf16x8 bv = b[mb];
+      if (NORM) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float xf = static_cast<float>(bv[e]);
+          ss[mb] += xf * xf;
+          bv[e] = static_cast<__bf16>(xf * gv[e]);
+        }
+      }
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[mb][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ct], bv, acc[mb][ct], 0, 0, 0);
+    }
+  }
+
+  // the waves' partial sums, over the stages (every wave is done reading them)
+  __builtin_amdgcn_s_barrier();
+  float(*red)[MB][CT][64][4] = reinterpret_cast<float(*)[MB][CT][64][4]>(lds);
+  float(*red_ss)[MB][16] = reinterpret_cast<float(*)[MB][16]>(lds + WAVES * MB * CT * 1024);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][mb][ct][lane][i] = acc[mb][ct][i];
+    if (NORM) {
+      float t = ss[mb];
+      t += __shfl_xor(t, 16, 64);
+      t += __shfl_xor(t, 32, 64);
+      if (g == 0) red_ss[wave][mb][c16] = t;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < TPW; ++j) {
+    const int t = j * WAVES + wave, mb = t / CT, ct = t % CT;
+    if (t >= TILES) continue;
+    const int n = n0 + ct * 16 + g * 4;      // the lane's four consecutive output columns
+    const int m = mb * 16 + c16;
+    if (m >= M) continue;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) s += red[w][mb][ct][lane][i];
+      v[i] = s;
+    }
+    if (NORM) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) s += red_ss[w][mb][c16];
+      const float mul = sqrtf((float)K) / (sqrtf(s) + eps);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= mul;
+    }
+    if (EPI == EPI_ROPE) {
+      if (n >= N) continue;
+      const int hd = rope.head_dim, half = hd / 2;
+      const int head = n / hd, e0 = n % hd;
+      const bool is_q = head < rope.n_heads, is_v = head >= rope.n_heads + rope.n_kv_heads;
+      float y[4] = {v[0], v[1], v[2], v[3]};
+      int d[4];
+      if (is_v) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) d[i] = e0 + i;
+      } else {
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          const int pair = e0 / 2 + jj;
+          d[2 * jj] = rope.interleaved ? 2 * pair : pair;
+          d[2 * jj + 1] = rope.interleaved ? 2 * pair + 1 : pair + half;
+          if (rope.table) {
+            const float x1 = v[2 * jj], x2 = v[2 * jj + 1];
+            y[2 * jj] = x1 * cs[j][jj].x - x2 * cs[j][jj].y;
+            y[2 * jj + 1] = x2 * cs[j][jj].x + x1 * cs[j][jj].y;
+          }
+        }
+      }
+      if (is_q) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) C[(long)m * c_ld + (long)head * hd + d[i]] = from_f<TO>(y[i]);
+      } else if (rope.write_cache) {
+        const int page = slot[j] / rope.page_size, off = slot[j] % rope.page_size;
+        const int kvh = is_v ? head - rope.n_heads - rope.n_kv_heads : head - rope.n_heads;
+        bf16* hp = rope.plane + (((long)page * 2 + (is_v ? 1 : 0)) * rope.n_kv_heads + kvh) * rope.page_size * hd;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (is_v) hp[(long)d[i] * rope.page_size + off] = static_cast<__bf16>(y[i]);
+          else hp[(long)off * hd + d[i]] = static_cast<__bf16>(y[i]);
+        }
+      }
+    } else if (EPI == EPI_SWIGLU) {
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) {
+        if (n + 2 * jj + 1 < N) {
+          const float gt = v[2 * jj], up = v[2 * jj + 1];
+          C[(long)m * c_ld + n / 2 + jj] = from_f<TO>(gt / (1.f + __expf(-gt)) * up);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (n + i < N) {
+          float s = v[i];
+          if (EPI == EPI_RESIDUAL) s += res[j][i];
+          C[(long)m * c_ld + n + i] = from_f<TO>(s);
+        }
+      }
+    }
+  }
+}
+
 // (these can be set from outside: the kernel tests make small matrices take the wide path, and measurements compare
 // panel heights)
 static int g_wide_tiles = 256;   // from this many 32-column workgroups on (one a compute unit), a workgroup takes two column tiles
-static int g_wide_max_blocks = 2;   // with up to two blocks of 16 rows
 TIS_EXPORT void tis_gemm_skinny_wide_tiles(int n_workgroups) { g_wide_tiles = n_workgroups; }
-TIS_EXPORT void tis_gemm_skinny_wide_max_blocks(int n) { g_wide_max_blocks = n; }
+static int g_staged_stages = 0;    // measurements: stages of LDS of the staged kernel, 2 or 4 (0: as chosen below)
+static int g_units = 256;          // compute units of the device: set by whoever knows (the default is an MI355X)
+TIS_EXPORT void tis_gemm_skinny_staged_stages(int stages) { g_staged_stages = stages; }
+TIS_EXPORT void tis_gemm_skinny_units(int n) { if (n > 0) g_units = n; }
 
+template <bool NORM, int EPI, typename TO>
+static int launch_staged(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
+                         void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope) {
+  // Panels of 32 rows: what a workgroup draws from L2 and HBM is what bounds it (about 50 GB/s), so small panels on
+  // many workgroups beat panels of 64 rows wherever they were measured (64 rows, 0.9B widths, us, panels of 32 / of
+  // 64: down 10.7 / 14.9, attention output 6.3 / 8.2, q/k/v 8.6 / 10.0, gate-up 11.2 / 11.7).
+  const int mb = 2;
+  const int panels = (M + mb * 16 - 1) / (mb * 16);
+  if (panels > 65535) return tis_fail("gemm_skinny: %d rows are more panels than a grid holds", M);
+  if (NORM && ((uintptr_t)gain % 16)) return tis_fail("gemm_skinny: the norm's gains must be 16-byte aligned");
+  // two column tiles a workgroup where that still leaves a workgroup for every compute unit: the panel's activations,
+  // which a workgroup copies in full, then serve twice as many weights
+  int ct = 1;
+  if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) {
+    if ((long)((N + 31) / 32) * panels >= g_wide_tiles) ct = 2;
+  }
+  const dim3 grid((N + 16 * ct - 1) / (16 * ct), panels);
+  // Stages of LDS: four (three chunks in flight) while every workgroup has a compute unit to itself; two, so that two
+  // or three workgroups share a unit, once there are more workgroups than units (gate-up at 64 rows: 11.2 us with
+  // two stages, 14.0 with four; down at 64 rows, 192 workgroups: 10.7 with four, 13.5 with two).
+  int ns = (long)grid.x * grid.y > g_units ? 2 : 4;
+  if (g_staged_stages) ns = g_staged_stages;
+#define STAGED(CTV, NS)                                                                                           \
+  if (ct == CTV && ns == NS) {                                                                                    \
+    gemm_staged_kernel<2, CTV, NORM, EPI, TO, NS><<<grid, 512, 0, stream>>>(                                      \
+        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);      \
+    return 0;                                                                                                     \
+  }
+  STAGED(1, 4) STAGED(1, 2)
+  if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) { STAGED(2, 4) STAGED(2, 2) }
+#undef STAGED
+  return tis_fail("gemm_skinny: no staged kernel for %d column tiles and %d stages", ct, ns);
+}
 
 template <bool NORM, int EPI, typename TO>
 static int launch(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
@@ -315,13 +628,11 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
   // half as wide column tiles where full ones would leave more than half of the 256 compute units idle and the
   // rows allow it (measured at N = 1536: 6.2 instead of 8.2 us for K = 4096, 4.1 instead of 4.8 us for K = 1536;
   // at N = 2304 with the norm in front the wider tile stays ahead, and a quarter tile never beat the half)
+  if (M > 16) return launch_staged<NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
   int r = (M <= 8 && (N + 15) / 16 <= 128) ? 2 : 1;
   if (r != 1 && r != 2) return tis_fail("gemm_skinny: %d chunks a step; 1 or 2 are built", r);
   if (r == 2 && M > 8) return tis_fail("gemm_skinny: %d rows do not fit 8 columns a workgroup", M);
-  // rows beyond a panel's go to further panels (blockIdx.y)
-  const int mb = M <= 16 ? 1 : 2;
-  const int panels = (M + mb * 16 - 1) / (mb * 16);
-  if (panels > 65535) return tis_fail("gemm_skinny: %d rows are more panels than a grid holds", M);
+  const int mb = 1, panels = 1;          // (more than 16 rows went to the staged kernel above)
   const int steps = (K + 32 * r - 1) / (32 * r);
   int waves, u;
   if (steps >= 24) {
@@ -332,13 +643,12 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
     waves = 4;
     u = (steps % 3 == 0 && steps % 4 != 0) || steps == 12 ? 3 : 4;
   }
-  if (mb > 1 && waves != 8) { waves = 8; u = 4; }   // two row blocks are built for eight waves only
   // two column tiles a workgroup where the matrix is wide enough to fill the chip with half as many workgroups:
   // the activations, the gains and the norm's arithmetic are then shared by twice as many weights (the gate-up
   // product of 8192 columns and the output table: 2.5 % of a decode step at batch 8)
   int ct = 1;
   if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) {
-    if (r == 1 && mb <= g_wide_max_blocks && waves == 8 && (N + 31) / 32 >= g_wide_tiles) ct = 2;
+    if (r == 1 && waves == 8 && (N + 31) / 32 >= g_wide_tiles) ct = 2;
   }
   const int cols = 16 / r * ct;
   const dim3 grid((N + cols - 1) / cols, panels);
@@ -349,7 +659,7 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
         (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);     \
     return 0;                                                                                                    \
   }
-    WIDE(1, 3) WIDE(1, 4) WIDE(2, 3) WIDE(2, 4)
+    WIDE(1, 3) WIDE(1, 4)
 #undef WIDE
   }
 #define CFG(MBV, WV, UV, RV)                                                                                     \
@@ -360,7 +670,6 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
   }
 #define CFGS(RV) CFG(1, 4, 3, RV) CFG(1, 4, 4, RV) CFG(1, 8, 3, RV) CFG(1, 8, 4, RV)
   CFGS(1) CFGS(2)
-  CFG(2, 8, 3, 1) CFG(2, 8, 4, 1)
 #undef CFGS
 #undef CFG
   return tis_fail("gemm_skinny: no kernel for %d row blocks, %d waves of %d steps and %d chunks", mb, waves, u, r);

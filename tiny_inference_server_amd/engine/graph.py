@@ -12,6 +12,8 @@ library chooses its algorithms for the shape then), so a capture records kernel 
 """
 from __future__ import annotations
 
+import gc
+
 import numpy as np
 import torch
 
@@ -55,8 +57,18 @@ class DecodeGraph:
         if capture:
             self.graph = torch.cuda.CUDAGraph()
             torch.cuda.synchronize(dev)
-            with torch.cuda.graph(self.graph):
-                self._launch()
+            # No garbage collection while the stream is capturing: a collection may finalise an engine that is no
+            # longer used (engines and their captured steps refer to each other, so only the collector frees them),
+            # and destroying its graphs in the middle of a capture aborts the process. The context below collects
+            # once before the capture begins.
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(self.graph):
+                    self._launch()
+            finally:
+                if collecting:
+                    gc.enable()
         self.copied.record()
         # what the quick update needs: which requests, in which order, the buffer holds, and where their arrays lie
         self.slots = tuple(e.slot for e in plan.entries)

@@ -110,7 +110,7 @@ def library(name: str) -> _Lib:
     return lib
 
 
-_FEW_ROWS = 64                  # up to this many rows a product goes to the few-row kernel whatever its widths
+_FEW_ROWS = 128                 # up to this many rows a product goes to the few-row kernels whatever its widths
 
 _WIDTHS_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "library_widths.json")
 
@@ -423,6 +423,7 @@ class HipOps:
         # compute units of this device: what the attention planner spreads waves over
         self.units = int(torch.cuda.get_device_properties(self.device).multi_processor_count) or _CHIP_UNITS
         if dtype == torch.bfloat16:
+            self.gemm_skinny.cdll.tis_gemm_skinny_units(self.units)
             self.gemm_library = library("gemm_library")
             with torch.cuda.device(self.device):
                 self.gemm_library.tis_gemm_library_init()

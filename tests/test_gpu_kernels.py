@@ -724,3 +724,14 @@ def test_sampling_with_the_context_kept_on_the_device(sampling_kernel, V):
             want = seen[lines[i]].clone(); want[by_table[i]] = 1
             assert torch.equal(after[lines[i]], want)
     assert torch.equal(after[[1, 4, 5, 7]], seen[[1, 4, 5, 7]])
+
+
+def test_the_measurement_tool_runs(capsys):
+    """python -m tiny_inference_server_amd.ops.kernel_bench, the tool that the counter profiles under profiles/ were
+    made with: one small case of each kind runs and prints its line."""
+    from tiny_inference_server_amd.ops.kernel_bench import main
+    assert main(["attention", "--segments", "100:1x3,0:40", "--heads", "4", "--kv-heads", "2", "--head-dim", "64", "--reps", "2"]) == 0
+    assert main(["product", "--rows", "8", "--out", "96", "--in", "64", "--kind", "norm+gate", "--reps", "2"]) == 0
+    assert main(["product", "--rows", "40", "--out", "96", "--in", "64", "--kind", "residual", "--copies", "3", "--reps", "2"]) == 0
+    out = capsys.readouterr().out
+    assert out.count(" us; ") == 3 and "attention 100:1x3,0:40" in out and "product residual rows 40" in out

@@ -142,7 +142,8 @@ class PlanningOps(TorchOps):
 def test_parts_plan_again_for_every_replay_of_a_captured_step():
     """A captured step of requests that differ widely in length carries a work list planned on the host. When the
     same requests come again the list is planned again, for the new positions, into its place in the step's buffer:
-    after every step the buffer holds, integer for integer, what a fresh plan of that step holds."""
+    what every step ran on (the device's copy of the buffer) is, integer for integer, what a fresh plan of that step
+    holds. (The host's copy is by then already filled for the step after, ahead of time: all but its tokens.)"""
     from tiny_inference_server_amd.engine.batch import Entry, first_stage_rows, plan_step_batch
     name = "D"
     folder = H.model_folder(name, "float32")
@@ -152,7 +153,7 @@ def test_parts_plan_again_for_every_replay_of_a_captured_step():
     eng = Engine(folder, dtype="float32", page_size=16, max_tokens=1024, max_requests=4, ops=PlanningOps(graphs=True))
     for rid, ids in reqs.items():
         eng.step([(rid, ids[:-24], [])])
-    main, checked = {}, 0
+    main, checked, ahead = {}, 0, 0
     for t in range(24):
         entries = [(rid, [ids[len(ids) - 24 + t]], [0]) for rid, ids in reqs.items()]
         slots = [(eng.requests[rid][0], eng.requests[rid][1]) for rid in reqs]
@@ -172,9 +173,12 @@ def test_parts_plan_again_for_every_replay_of_a_captured_step():
         assert fresh.layout() == graph.layout
         want = torch.zeros_like(graph.host)
         fresh.packer.fill(want)
-        assert torch.equal(graph.host[:fresh.packer.total], want[:fresh.packer.total]), t
+        assert torch.equal(graph.dev[:fresh.packer.total].cpu(), want[:fresh.packer.total]), t
+        if graph._ahead is not None:            # (not after the step that made the graph)
+            assert graph._ahead[0].tolist() == [fed + 1 for _, fed in slots]
+            ahead += 1
         checked += 1
-    assert checked >= 20 and eng.graph_replays >= 20
+    assert checked >= 20 and eng.graph_replays >= 20 and ahead >= 18
     H.compare_with_plain(folder, reqs, main, {}, TOL["float32"] * scale_of(folder, reqs), 0)
 
 

@@ -86,6 +86,7 @@ class DecodeGraph:
         self.extras_at = [[(off(i), plan.packer.offsets[i][1]) for i in sorted(v[0] for v in pl["extra"].values())]
                           for pl in plan.plans]
         self.extras_host = [tuple(sorted((k, v[1:]) for k, v in pl["extra"].items())) for pl in plan.plans]
+        self._ahead = None       # (positions the buffer was filled for ahead of time, requests still to be filled)
 
     def _launch(self):
         engine, n = self.engine, self.step.n_wanted
@@ -104,32 +105,70 @@ class DecodeGraph:
 
     def run_same_requests(self, entries) -> torch.Tensor:
         """The next step of the very requests whose arrays the buffer already holds, in the same order: only
-        tokens, positions, write slots and newly taken pages change, and those are written in place."""
+        tokens, positions, write slots and newly taken pages change, and those are written in place.
+
+        Everything but the tokens depends on the requests' positions alone, and after a step of single tokens the
+        likeliest next step is the same requests one position on. So once a step has been launched, while the GPU
+        runs it (the caller cannot go on before it has the step's tokens anyway), the buffer is filled for that next
+        step; when it comes, only its tokens, and the lines of requests that have taken a page since, are left to
+        write before the copy and the replay."""
         self.copied.synchronize()
         flat = self.host.numpy()
         n = len(entries)
         starts = np.fromiter((e.start for e in entries), dtype=np.int64, count=n)
         tokens = np.fromiter((e.tokens[0] for e in entries), dtype=np.int32, count=n)
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None and len(ahead[0]) == n and np.array_equal(ahead[0], starts):
+            if len(ahead[1]):
+                self._fill_positions(flat, starts, only=ahead[1])
+        else:
+            self._fill_positions(flat, starts)
+        for st in self.stage_at:
+            flat[st["tokens"]:st["tokens"] + n] = tokens
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+        self._replay()
+        # the buffer for the step after this one, while this one runs (the copy above has to have left the buffer)
+        self.copied.synchronize()
+        nxt = starts + 1
+        if self.cache.spare_slot is not None:       # (lines that fill the step up stay where they are)
+            nxt = nxt - np.fromiter((s == self.cache.spare_slot for s in self.slots), dtype=np.int64, count=n)
+        self._ahead = (nxt, self._fill_positions(flat, nxt, ahead=True))
+        return self.logits
+
+    def _fill_positions(self, flat, starts, only=None, ahead=False):
+        """Positions, write slots, newly taken pages and the parts' work lists for requests that stand at `starts`.
+        only: the indices of the requests whose lines are to be written (the others' are right already).
+        ahead: the step has not come yet, so a request whose position opens a page may not have that page; such
+        requests are skipped and their indices returned, to be filled when the step comes."""
+        n = len(starts)
         ps = self.page_size
+        late = np.zeros(0, dtype=np.int64)
         for g, (t_off, (rows, width)) in self.table_at.items():
             tables = self.cache.groups[g].tables
             need = starts // ps + 1
             for k in np.nonzero(need > self.pages_held[g])[0]:
                 t = tables[self.slots[k]]
+                if len(t) < need[k]:
+                    if not ahead:
+                        raise RuntimeError("a request's position lies beyond its pages")
+                    late = np.union1d(late, [k])
+                    continue
                 if len(t) > width:
                     raise RuntimeError("a block table outgrew the captured width")
                 flat[t_off + k * width:t_off + k * width + len(t)] = [p if p >= 0 else 0 for p in t]
                 self.pages_held[g][k] = len(t)
-        rows_idx = np.arange(n)
+        which = np.arange(n) if only is None else np.asarray(only, dtype=np.int64)
+        if ahead and len(late):
+            which = np.setdiff1d(which, late)
         for st in self.stage_at:
-            pos = starts - st["lag"]
-            flat[st["tokens"]:st["tokens"] + n] = tokens
-            flat[st["positions"]:st["positions"] + n] = pos
+            pos = starts[which] - st["lag"]
+            flat[st["positions"] + which] = pos
             for g, w_off in st["ws"].items():
                 t_off, (rows, width) = self.table_at[g]
                 table = flat[t_off:t_off + rows * width].reshape(rows, width)
-                flat[w_off:w_off + n] = table[rows_idx, pos // ps] * ps + pos % ps
-        if any(self.extras_at):
+                flat[w_off + which] = table[which, pos // ps] * ps + pos % ps
+        if only is None and any(self.extras_at):
             # the parts plan again for the new positions, into the places their arrays have in the buffer
             for at, host_values, st in zip(self.extras_at, self.extras_host, self.stage_at):
                 slots_left = list(at)
@@ -146,15 +185,13 @@ class DecodeGraph:
                 extra = self.engine.model.plan_rows([(k, int(pos[k]), 1) for k in range(n)], put, self.mode)
                 if slots_left or tuple(sorted((k, v[1:]) for k, v in extra.items())) != host_values:
                     raise RuntimeError("the parts' planning no longer fits the captured step")
-        self.dev.copy_(self.host, non_blocking=True)
-        self.copied.record()
-        self._replay()
-        return self.logits
+        return late
 
     def run(self, plan: StepPlan, occupants=None) -> torch.Tensor:
         if plan.layout() != self.layout:
             raise RuntimeError("this step's arrays do not have the captured layout")
         self.copied.synchronize()            # the previous copy out of the pinned buffer has finished
+        self._ahead = None
         plan.packer.fill(self.host)
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()

@@ -672,10 +672,11 @@ def test_projection_with_rotary_and_cache_write(ops_for, dtype, M, n_heads, n_kv
         torch.testing.assert_close(got.double().view(M, n_heads, hd), q * c + rot * s, **t)
 
 
-@pytest.mark.parametrize("M", [1, 8, 16])
+@pytest.mark.parametrize("M", [1, 8, 16, 20, 40, 70])
 def test_skinny_product_with_two_column_tiles_a_workgroup(ops_for, M):
-    """Very wide matrices give a workgroup two column tiles. Forced here at a small width that ends inside the
-    second tile, for the plain, the 32-bit and the normed and gated product."""
+    """Very wide matrices give a workgroup two column tiles, in the kernel for up to 16 rows and in the staged one for
+    more. Forced here at a small width that ends inside the second tile, for the plain, the 32-bit and the normed and
+    gated product; the staged kernel also with two stages of LDS instead of four."""
     ops, ref = ops_for(torch.bfloat16), TorchOps(dtype=torch.bfloat16)
     N, K = 138, 800
     x, w = rnd((M, K), torch.bfloat16, 91, 2.0), rnd((N, K), torch.bfloat16, 92, K ** -0.5)
@@ -686,10 +687,15 @@ def test_skinny_product_with_two_column_tiles_a_workgroup(ops_for, M):
     try:
         wide = [ops.linear(x.cuda(), w.cuda()).cpu(), ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32).cpu(),
                 ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()]
+        ops.gemm_skinny.cdll.tis_gemm_skinny_staged_stages(2)
+        wide2 = [ops.linear(x.cuda(), w.cuda()).cpu(), ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32).cpu(),
+                 ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()]
     finally:
         ops.gemm_skinny.cdll.tis_gemm_skinny_wide_tiles(256)
-    for a, b in zip(narrow, wide):
+        ops.gemm_skinny.cdll.tis_gemm_skinny_staged_stages(0)
+    for a, b, c in zip(narrow, wide, wide2):
         assert torch.equal(a, b)          # the same sums in the same order, only spread over workgroups differently
+        assert torch.equal(a, c)
     torch.testing.assert_close(wide[1].double(), x.double() @ w.double().t(), rtol=1e-4, atol=1e-4)
 
 

@@ -577,10 +577,13 @@ def test_product_with_norm_residual_and_gate_for_many_rows(ops_for, M, N, K):
     torch.testing.assert_close(ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), want,
                                rtol=3e-2, atol=3e-2)
     if (N, K) not in ops.library_widths or M <= ops.few_rows:
-        # the few-row kernel: a row's result does not depend on its panel or on the other rows
+        # our own kernels: a row's result does not depend on its panel or on the other rows
         for r in (0, M // 2, M - 1):
-            alone = ops.linear(x[r:r + 1].cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()
-            assert torch.equal(alone[0], normed[r])
+            others = rnd((M, K), torch.bfloat16, 84, 3.0)
+            shift = (M // 3) if r + M // 3 < M else 0             # the row moves to another panel where it can
+            others[r + shift] = x[r]
+            again = ops.linear(others.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()
+            assert torch.equal(again[r + shift], normed[r])
 
 
 def test_library_product_at_listed_widths(ops_for):
@@ -630,9 +633,19 @@ def test_skinny_product_with_fused_norm_residual_and_gate(ops_for, M, N, K):
     torch.testing.assert_close(lg.cpu().double(), x.double() @ w.double().t(), rtol=1e-4, atol=1e-4)   # 32-bit sums kept
     want = torch.nn.functional.silu(normed[:, 0::2]) * normed[:, 1::2]
     torch.testing.assert_close(ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu().double(), want, **t)
-    # a row's result does not depend on the other rows of the batch
-    alone = ops.linear(x[:1].cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()
-    assert torch.equal(alone[0], ops.linear(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()[0])
+    # a row's result does not depend on the other rows of the batch, nor on which row of it it is
+    both = ops.linear(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()
+    others = rnd((M, K), torch.bfloat16, 84, 3.0)
+    others[M - 1] = x[0]
+    assert torch.equal(ops.linear(others.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()[M - 1], both[0])
+    # and the two kernels (few rows of a narrow matrix; everything else) agree up to the order of their sums
+    ops.gemm_skinny.cdll.tis_gemm_skinny_staged_always(1)
+    try:
+        staged = ops.linear(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()
+    finally:
+        ops.gemm_skinny.cdll.tis_gemm_skinny_staged_always(0)
+    torch.testing.assert_close(staged.double(), normed, **t)
+    torch.testing.assert_close(staged.float(), both.float(), rtol=8e-3, atol=2e-3)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -674,17 +687,18 @@ def test_projection_with_rotary_and_cache_write(ops_for, dtype, M, n_heads, n_kv
 
 @pytest.mark.parametrize("M", [1, 8, 16, 20, 40, 70])
 def test_skinny_product_with_two_column_tiles_a_workgroup(ops_for, M):
-    """Very wide matrices give a workgroup two column tiles, in the kernel for up to 16 rows and in the staged one for
-    more. Forced here at a small width that ends inside the second tile, for the plain, the 32-bit and the normed and
-    gated product; the staged kernel also with two stages of LDS instead of four."""
+    """Very wide matrices give a workgroup of the staged kernel two column tiles. Forced here at a small width that
+    ends inside the second tile, for the plain, the 32-bit and the normed and gated product, with one and with two
+    blocks of 16 rows, and with two stages of LDS instead of four."""
     ops, ref = ops_for(torch.bfloat16), TorchOps(dtype=torch.bfloat16)
     N, K = 138, 800
     x, w = rnd((M, K), torch.bfloat16, 91, 2.0), rnd((N, K), torch.bfloat16, 92, K ** -0.5)
     gain = 1 + 0.1 * rnd((K,), torch.float32, 93)
-    narrow = [ops.linear(x.cuda(), w.cuda()).cpu(), ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32).cpu(),
-              ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()]
-    ops.gemm_skinny.cdll.tis_gemm_skinny_wide_tiles(1)
+    ops.gemm_skinny.cdll.tis_gemm_skinny_staged_always(1)
     try:
+        narrow = [ops.linear(x.cuda(), w.cuda()).cpu(), ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32).cpu(),
+                  ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()]
+        ops.gemm_skinny.cdll.tis_gemm_skinny_wide_tiles(1)
         wide = [ops.linear(x.cuda(), w.cuda()).cpu(), ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32).cpu(),
                 ops.linear_swiglu(x.cuda(), w.cuda(), rms=(gain.cuda(), 1e-5)).cpu()]
         ops.gemm_skinny.cdll.tis_gemm_skinny_staged_stages(2)
@@ -693,6 +707,7 @@ def test_skinny_product_with_two_column_tiles_a_workgroup(ops_for, M):
     finally:
         ops.gemm_skinny.cdll.tis_gemm_skinny_wide_tiles(256)
         ops.gemm_skinny.cdll.tis_gemm_skinny_staged_stages(0)
+        ops.gemm_skinny.cdll.tis_gemm_skinny_staged_always(0)
     for a, b, c in zip(narrow, wide, wide2):
         assert torch.equal(a, b)          # the same sums in the same order, only spread over workgroups differently
         assert torch.equal(a, c)

@@ -1,16 +1,21 @@
 // C[M,N] = f(A[M,K]) . W[N,K]^T for few rows: the matrix product of decode steps, where the job is to stream W from
-// HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950). Two kernels: up to 16 rows, operands straight from memory into
-// registers (below); from 17 rows on, operands staged through LDS, in panels of 32 rows, one per blockIdx.y, each an
-// independent product over the same weights (the panels of a column tile run side by side, so the weights come from
-// HBM once and from the caches after that). That is right for a few panels; for many, every panel streams all of W
-// again, which only a product tiled in both directions avoids: it still gives the right result, slowly.
+// HBM once, on v_mfma_f32_16x16x32_bf16 (gfx950). Two kernels. The first (below) takes up to 8 rows against a
+// matrix of up to 2,048 rows: operands go straight from memory into registers and a workgroup owns only 8 output
+// columns, so that a narrow matrix still gives a workgroup to every compute unit. The staged kernel (further down)
+// takes everything else: operands pass through LDS by direct loads, in panels of 16 or 32 rows of X, one per
+// blockIdx.y, each an independent product over the same weights (the panels of a column tile run side by side, so
+// the weights come from HBM once and from the caches after that). That is right for a few panels; for many, every
+// panel streams all of W again, which only a product tiled in both directions avoids: it still gives the right
+// result, slowly. Measured on MI355X (microseconds, first kernel / staged): at 8 rows the 1536x1536 product 4.8 / 5.0
+// and the 1536x4096 one 7.3 / 8.2, but 2304x1536 6.3 / 5.5, 8192x1536 8.2 / 7.2, the 147 MB output table 35.5 / 30.4;
+// at 16 rows the staged kernel wins everywhere (8192x1536: 8.7 / 7.3, 1536x4096: 10.5 / 8.4).
 //
-// The kernel for up to 16 rows:
-// One workgroup owns 16 rows of W (16 output columns; 8 in the narrow variant below) over the whole of K; its
-// waves take the 32-wide steps of K in turn, so together they read each weight row in contiguous runs. W rows are the A operand straight from
-// global memory (16 bytes per lane), the activations are the B operand straight from L2 (they are a few KB
-// and every workgroup reads the same ones), so no LDS is used for operands. Partial sums of the waves are
-// added through LDS in a fixed order: a row's result does not depend on M or on the other rows.
+// The first kernel:
+// One workgroup owns 16 rows of W (16 output columns; 8 in the variant that is built, see R below) over the whole of
+// K; its waves take the 32-wide steps of K in turn, so together they read each weight row in contiguous runs. W rows
+// are the A operand straight from global memory (16 bytes per lane), the activations are the B operand straight
+// from L2 (they are a few KB and every workgroup reads the same ones), so no LDS is used for operands. Partial sums
+// of the waves are added through LDS in a fixed order: a row's result does not depend on M or on the other rows.
 //
 // Fused around the product, so that a layer needs fewer launches and no round trips for small tensors:
 //   NORM      the reference's RMSNorm of the input rows (main_models_new.py:38-42): the activations are multiplied
@@ -53,12 +58,10 @@ struct RopeArgs {
 // of eight steps, or sixteen waves, so that all of a wave's loads are in flight at once, measured the same within
 // noise (the gated product at 64 rows slower: fewer workgroups fit a compute unit).
 //
-// MB: blocks of 16 rows of X that share every weight tile a wave loads. One is built: with two, a wave fetches its
-// own pieces of twice the activations, 16 bytes a lane from 16 different rows, and that is what its time went to
-// (down product, 12.6 MB: 7.3 us at 8 rows, 10.4 at 16, 14.7 at 32); 17 rows and more go to the staged kernel.
-//
-// CT: column tiles of 16 a workgroup owns. Two where the matrix is so wide that half as many workgroups still fill
-// the chip: a wave then uses the activations it loaded (and normed) for twice as many weights.
+// MB: blocks of 16 rows of X that share every weight tile a wave loads, and CT: column tiles of 16 a workgroup
+// owns. One of each is built. With two row blocks a wave fetches its own pieces of twice the activations, 16 bytes a
+// lane from 16 different rows, and that is what its time went to (down product, 12.6 MB: 7.3 us at 8 rows, 10.4 at
+// 16, 14.7 at 32); with two column tiles the staged kernel is faster for the same shapes.
 //
 // R: with 16 output columns per workgroup a matrix of 1536 rows gives 96 workgroups, and a compute unit draws
 // only about 24 GB/s, so the 160 idle units cost more than the product. For M <= 16/R rows a workgroup
@@ -299,10 +302,11 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_skinny_kernel(
   }
 }
 
-// ---- 17 rows and more: operands staged through LDS ----
+// ---- the staged kernel: operands through LDS ----
 //
-// From two blocks of rows on, what a workgroup of the kernel above spends its time on is the activations: every wave
-// fetches its own pieces of X, 16 bytes a lane from 16 different rows, and of W likewise. Here a workgroup of eight waves
+// What a workgroup of the kernel above spends its time on, as soon as it has more than a few rows or columns, is
+// the waiting for its own loads: every wave fetches its pieces of X, 16 bytes a lane from 16 different rows, and of
+// W likewise, into registers it must hold until the products. Here a workgroup of eight waves
 // owns CT * 16 columns and a panel of MB * 16 rows over the whole of K and walks K in chunks of 256: a chunk's
 // weight rows and activation rows (512 bytes each) are copied into LDS by loads that write LDS directly
 // (global_load_lds_dwordx4: no registers; a wave's load is two whole 512-byte runs), NSTAGE - 1 chunks ahead of the
@@ -584,6 +588,8 @@ __global__ __launch_bounds__(512) void gemm_staged_kernel(
 static int g_wide_tiles = 256;   // from this many 32-column workgroups on (one a compute unit), a workgroup takes two column tiles
 TIS_EXPORT void tis_gemm_skinny_wide_tiles(int n_workgroups) { g_wide_tiles = n_workgroups; }
 static int g_staged_stages = 0;    // measurements: stages of LDS of the staged kernel, 2 or 4 (0: as chosen below)
+static int g_staged_always = 0;    // measurements and tests: the staged kernel also where the first one would be chosen
+TIS_EXPORT void tis_gemm_skinny_staged_always(int on) { g_staged_always = on; }
 static int g_units = 256;          // compute units of the device: set by whoever knows (the default is an MI355X)
 TIS_EXPORT void tis_gemm_skinny_staged_stages(int stages) { g_staged_stages = stages; }
 TIS_EXPORT void tis_gemm_skinny_units(int n) { if (n > 0) g_units = n; }
@@ -591,10 +597,10 @@ TIS_EXPORT void tis_gemm_skinny_units(int n) { if (n > 0) g_units = n; }
 template <bool NORM, int EPI, typename TO>
 static int launch_staged(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
                          void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope) {
-  // Panels of 32 rows: what a workgroup draws from L2 and HBM is what bounds it (about 50 GB/s), so small panels on
+  // Up to 16 rows one block of rows; beyond, panels of 32 rows: what a workgroup draws from L2 and HBM is what bounds it (about 50 GB/s), so small panels on
   // many workgroups beat panels of 64 rows wherever they were measured (64 rows, 0.9B widths, us, panels of 32 / of
   // 64: down 10.7 / 14.9, attention output 6.3 / 8.2, q/k/v 8.6 / 10.0, gate-up 11.2 / 11.7).
-  const int mb = 2;
+  const int mb = M <= 16 ? 1 : 2;
   const int panels = (M + mb * 16 - 1) / (mb * 16);
   if (panels > 65535) return tis_fail("gemm_skinny: %d rows are more panels than a grid holds", M);
   if (NORM && ((uintptr_t)gain % 16)) return tis_fail("gemm_skinny: the norm's gains must be 16-byte aligned");
@@ -610,14 +616,14 @@ static int launch_staged(const void* X, long x_ld, const void* W, const float* g
   // two stages, 14.0 with four; down at 64 rows, 192 workgroups: 10.7 with four, 13.5 with two).
   int ns = (long)grid.x * grid.y > g_units ? 2 : 4;
   if (g_staged_stages) ns = g_staged_stages;
-#define STAGED(CTV, NS)                                                                                           \
-  if (ct == CTV && ns == NS) {                                                                                    \
-    gemm_staged_kernel<2, CTV, NORM, EPI, TO, NS><<<grid, 512, 0, stream>>>(                                      \
+#define STAGED(MBV, CTV, NS)                                                                                      \
+  if (mb == MBV && ct == CTV && ns == NS) {                                                                       \
+    gemm_staged_kernel<MBV, CTV, NORM, EPI, TO, NS><<<grid, 512, 0, stream>>>(                                    \
         (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);      \
     return 0;                                                                                                     \
   }
-  STAGED(1, 4) STAGED(1, 2)
-  if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) { STAGED(2, 4) STAGED(2, 2) }
+  STAGED(2, 1, 4) STAGED(2, 1, 2) STAGED(1, 1, 4) STAGED(1, 1, 2)
+  if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) { STAGED(2, 2, 4) STAGED(2, 2, 2) STAGED(1, 2, 4) STAGED(1, 2, 2) }
 #undef STAGED
   return tis_fail("gemm_skinny: no staged kernel for %d column tiles and %d stages", ct, ns);
 }
@@ -625,14 +631,15 @@ static int launch_staged(const void* X, long x_ld, const void* W, const float* g
 template <bool NORM, int EPI, typename TO>
 static int launch(const void* X, long x_ld, const void* W, const float* gain, float eps, const void* R, long r_ld,
                   void* C, long c_ld, int M, int N, int K, hipStream_t stream, RopeArgs rope = RopeArgs()) {
-  // half as wide column tiles where full ones would leave more than half of the 256 compute units idle and the
-  // rows allow it (measured at N = 1536: 6.2 instead of 8.2 us for K = 4096, 4.1 instead of 4.8 us for K = 1536;
-  // at N = 2304 with the norm in front the wider tile stays ahead, and a quarter tile never beat the half)
-  if (M > 16) return launch_staged<NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
-  int r = (M <= 8 && (N + 15) / 16 <= 128) ? 2 : 1;
-  if (r != 1 && r != 2) return tis_fail("gemm_skinny: %d chunks a step; 1 or 2 are built", r);
-  if (r == 2 && M > 8) return tis_fail("gemm_skinny: %d rows do not fit 8 columns a workgroup", M);
-  const int mb = 1, panels = 1;          // (more than 16 rows went to the staged kernel above)
+  // Which kernel. Up to 8 rows of a matrix of at most 2,048 rows (the attention output and down products) the first
+  // kernel, with 8 columns a workgroup: twice the workgroups of 16-column tiles, where those would leave more than
+  // half of the 256 compute units idle (N = 1536: 6.2 instead of 8.2 us for K = 4096, 4.1 instead of 4.8 for K = 1536;
+  // the staged kernel there: 8.2 and 5.0). Everything else the staged kernel, which from 9 rows on, and for wider
+  // matrices at any row count, is the faster one (0.9B widths, 8 rows, us, first / staged: gate-up 8.2 / 7.2, q/k/v
+  // 6.3 / 5.5, output table 35.5 / 30.4; 16 rows: gate-up 8.7 / 7.3, down 10.5 / 8.4, q/k/v 6.7 / 5.5).
+  const bool narrow = M <= 8 && (N + 15) / 16 <= 128 && !g_staged_always;
+  if (!narrow) return launch_staged<NORM, EPI, TO>(X, x_ld, W, gain, eps, R, r_ld, C, c_ld, M, N, K, stream, rope);
+  constexpr int r = 2;
   const int steps = (K + 32 * r - 1) / (32 * r);
   int waves, u;
   if (steps >= 24) {
@@ -643,36 +650,16 @@ static int launch(const void* X, long x_ld, const void* W, const float* gain, fl
     waves = 4;
     u = (steps % 3 == 0 && steps % 4 != 0) || steps == 12 ? 3 : 4;
   }
-  // two column tiles a workgroup where the matrix is wide enough to fill the chip with half as many workgroups:
-  // the activations, the gains and the norm's arithmetic are then shared by twice as many weights (the gate-up
-  // product of 8192 columns and the output table: 2.5 % of a decode step at batch 8)
-  int ct = 1;
-  if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) {
-    if (r == 1 && waves == 8 && (N + 31) / 32 >= g_wide_tiles) ct = 2;
-  }
-  const int cols = 16 / r * ct;
-  const dim3 grid((N + cols - 1) / cols, panels);
-  if constexpr (EPI == EPI_NONE || EPI == EPI_SWIGLU) {
-#define WIDE(MBV, UV)                                                                                            \
-  if (ct == 2 && mb == MBV && u == UV) {                                                                         \
-    gemm_skinny_kernel<MBV, NORM, EPI, TO, 8, UV, 1, 2><<<grid, 8 * 64, 0, stream>>>(                            \
+  const dim3 grid((N + 16 / r - 1) / (16 / r), 1);
+#define CFG(WV, UV)                                                                                              \
+  if (waves == WV && u == UV) {                                                                                  \
+    gemm_skinny_kernel<1, NORM, EPI, TO, WV, UV, r, 1><<<grid, WV * 64, 0, stream>>>(                            \
         (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);     \
     return 0;                                                                                                    \
   }
-    WIDE(1, 3) WIDE(1, 4)
-#undef WIDE
-  }
-#define CFG(MBV, WV, UV, RV)                                                                                     \
-  if (ct == 1 && mb == MBV && waves == WV && u == UV && r == RV) {                                               \
-    gemm_skinny_kernel<MBV, NORM, EPI, TO, WV, UV, RV, 1><<<grid, WV * 64, 0, stream>>>(                         \
-        (const bf16*)X, x_ld, (const bf16*)W, gain, eps, (const bf16*)R, r_ld, (TO*)C, c_ld, M, N, K, rope);     \
-    return 0;                                                                                                    \
-  }
-#define CFGS(RV) CFG(1, 4, 3, RV) CFG(1, 4, 4, RV) CFG(1, 8, 3, RV) CFG(1, 8, 4, RV)
-  CFGS(1) CFGS(2)
-#undef CFGS
+  CFG(4, 3) CFG(4, 4) CFG(8, 3) CFG(8, 4)
 #undef CFG
-  return tis_fail("gemm_skinny: no kernel for %d row blocks, %d waves of %d steps and %d chunks", mb, waves, u, r);
+  return tis_fail("gemm_skinny: no kernel for %d waves of %d steps", waves, u);
 }
 
 template <bool NORM, int EPI, typename TO>

@@ -110,6 +110,8 @@ def product_case(ops, a):
         ops.few_rows = a.few_rows
     if a.staged:
         ops.gemm_skinny.cdll.tis_gemm_skinny_staged_stages(int(a.staged))
+    if a.staged_always:
+        ops.gemm_skinny.cdll.tis_gemm_skinny_staged_always(1)
     us = graph_time(kinds[a.kind], a.reps)
     print(f"product {a.kind} rows {m} out {n} in {k}: {us:.2f} us; weights {n * k * 2 / 1e6:.1f} MB -> "
           f"{n * k * 2 / us / 1e6:.2f} TB/s; {2 * m * n * k / us / 1e6:.1f} TFLOP/s")
@@ -138,6 +140,7 @@ def main(argv=None) -> int:
     pr.add_argument("--kind", choices=["plain", "residual", "norm", "norm+gate", "logits"], default="plain")
     pr.add_argument("--copies", type=int, default=1, help="weight matrices that the launches take in turn")
     pr.add_argument("--staged", default="", help="LDS stages of the few-row kernel for 17 rows and more: 2 or 4 (default: its own choice)")
+    pr.add_argument("--staged-always", action="store_true", help="that kernel also for up to 8 rows of narrow matrices")
     pr.add_argument("--few-rows", type=int, default=0, help="the row count up to which the few-row kernel is used (0: as built)")
     for p in (at, pr):
         p.add_argument("--reps", type=int, default=20)

@@ -55,6 +55,13 @@ __device__ __forceinline__ float column_max(float v) {
   auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
+// the largest of three numbers that are not NaN payloads to be quieted: one instruction (fmaxf would first copy each
+// operand through a maximum with itself)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 __device__ __forceinline__ float column_sum(float v) {
   auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
@@ -466,69 +473,92 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   const long k_head = (long)kvh * page_size * HD;
   const long v_head = ((long)n_kv_heads + kvh) * page_size * HD;
 
+  // No running maximum yet: a finite number far below any score, so that differences with it stay numbers (a
+  // column none of whose keys has counted so far keeps it, with a sum of zero; the merge gives such a part no weight)
+  constexpr float NO_MAX = -1e30f;
   f32x4 o[NB][DB];
   float m[NB], l[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
-    m[nb] = -INFINITY;
+    m[nb] = NO_MAX;
     l[nb] = 0.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db) o[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
 
-  // Page ids: every wave keeps, in a line of LDS of its own, the pages of a run of 64 16-key tiles (32 steps),
-  // fetched by one vector load a run; a step reads its two from there. (Fetched step by step they would be scalar
-  // loads, and the waits for LDS data wait for outstanding scalar loads as well: a round trip to memory every step.)
-  __shared__ int run_pages[TW][64];
+  // What the loop below spends per step is instructions, of any kind: a wave issues one every four cycles at best,
+  // and the matrix instructions of the other wave on its SIMD do not hide the rest. So whatever a step can know in
+  // advance is worked out here, once, as ranges of steps:
+  //   mine:   steps with a key that some row of this wave sees (others are skipped: past its last row, before its
+  //           first window)
+  //   free:   steps all of whose keys every row of the wave sees (no masking)
+  //   inside: steps all of whose keys some row of the tile sees (their values need no guarding, see `values`)
+  const int mine_lo = max(s_begin, (w_lo - k_lo) >> 5), mine_hi = active ? min(s_end, ((p_last - k_lo) >> 5) + 1) : 0;
+  const int free_lo = (lo_last - k_lo + 31) >> 5, free_hi = (p_first + 1 - k_lo) >> 5;
+  const int in_lo = (t_lo - k_lo + 31) >> 5, in_hi = (tp_last + 1 - k_lo) >> 5;
+
+  // Where a step's keys and values lie: every wave keeps, in a line of LDS of its own, the addresses of a run of 64
+  // 16-key tiles (32 steps), worked out by one lane each from one vector load a run; a step reads its two from there.
+  // (Fetched step by step the page ids would be scalar loads, and the waits for LDS data wait for outstanding scalar
+  // loads as well: a round trip to memory every step.) A tile past the request's keys, or on a page that a window
+  // has passed and given back (-1 in the table), reads page 0, which is always mapped; its scores are masked below,
+  // and so are its values.
+  struct TileAddress { const bf16* keys; const bf16* values; };      // of slot 0 of kv head 0, element 0
+  __shared__ __attribute__((aligned(16))) TileAddress run_tiles[TW][64];
   int run_first = s_begin;
   auto load_run = [&](int s0) {
     const int key0 = k_lo + (2 * s0 + lane) * 16;
-    run_pages[wave][lane] = bt[key0 < k_hi ? (PS16 ? key0 >> 4 : key0 / page_size) : 0];
+    const int pg = bt[key0 < k_hi ? (PS16 ? key0 >> 4 : key0 / page_size) : 0];
+    const bf16* page = plane + (long)(key0 < k_hi && pg >= 0 ? pg : 0) * page_stride;
+    const int slot0 = PS16 ? 0 : key0 % page_size;
+    run_tiles[wave][lane] = TileAddress{page + (long)slot0 * HD, page + slot0};
     run_first = s0;
   };
 
-  // A lane's pieces of a step as offsets inside a page: they never change. With a head size in steps of 32 all
-  // pieces of a fetch lie in the same 16-key tile, and the page's address is scalar.
+  // A lane's pieces of a step as offsets from those addresses: they never change. With a head size in steps of 32
+  // all pieces of a fetch lie in the same 16-key tile, and the address is scalar.
   constexpr bool T_UNIFORM = HD % 32 == 0;
+  constexpr bool T_IS_J = 2 * HD == TW * 64;     // fetch j holds the pieces of tile j
   unsigned k_off[TPT], v_off[TPT];       // in elements; less than a page
   int piece_t[TPT];
 #pragma unroll
   for (int j = 0; j < TPT; ++j) {
     const int c = tid + j * (TW * 64);                      // the piece's index in LDS
     const int t = c / (2 * HD);                             // keys and values alike
-    piece_t[j] = T_UNIFORM ? __builtin_amdgcn_readfirstlane(t) : t;
+    piece_t[j] = T_IS_J ? j : T_UNIFORM ? __builtin_amdgcn_readfirstlane(t) : t;
     k_off[j] = (unsigned)k_head + (c & 15) * HD + ((c >> 4) % NCH) * 8;
     v_off[j] = (unsigned)v_head + (((c >> 5) % DB) * 16 + (c & 15)) * page_size + ((c >> 4) & 1) * 8;
   }
 
-  // A step on its way from the pages to LDS buffer `buf`. A 16-key tile past the tile's keys reads page 0 (always
-  // mapped); its scores are masked below, and so are its values (see `values`).
+  // A step on its way from the pages to LDS buffer `buf`.
   auto stage = [&](int s, int buf) {
     if (s - run_first >= 32) load_run(s);
-    long kbase[2], vbase[2];  // offsets from the plane, so that every load below is plainly one from global memory
-    const int2 pages = *reinterpret_cast<const int2*>(&run_pages[wave][2 * (s - run_first)]);
+    const TileAddress* at = &run_tiles[wave][2 * (s - run_first)];
+    const bf16 *kbase[2], *vbase[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const int key0 = k_lo + s * 32 + t * 16;
-      const int pg = __builtin_amdgcn_readfirstlane(t ? pages.y : pages.x);
-      // (a page that a window has passed and given back reads as -1 in the table: page 0 stands in, masked like
-      // a tile past the keys)
-      const long page = (long)(key0 < k_hi && pg >= 0 ? pg : 0) * page_stride;
-      const int slot0 = PS16 ? 0 : key0 % page_size;
-      kbase[t] = page + (long)slot0 * HD;
-      vbase[t] = page + slot0;
+      if (T_UNIFORM) {
+        const uint64_t ka = (uint64_t)at[t].keys, va = (uint64_t)at[t].values;
+        kbase[t] = (const bf16*)(((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(ka >> 32)) << 32) |
+                                 (unsigned)__builtin_amdgcn_readfirstlane((int)ka));
+        vbase[t] = (const bf16*)(((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(va >> 32)) << 32) |
+                                 (unsigned)__builtin_amdgcn_readfirstlane((int)va));
+      } else {
+        kbase[t] = at[t].keys;
+        vbase[t] = at[t].values;
+      }
     }
 #pragma unroll
     for (int j = 0; j < TPT; ++j) {
       if (TCH % (TW * 64) != 0 && wave * 64 + j * (TW * 64) >= TCH) break;
-      if (T_UNIFORM) copy_to_lds(plane + kbase[piece_t[j]], k_off[j] * 2, &k_lds[buf][(wave + j * TW) * 512]);
-      else copy_to_lds(plane + (kbase[piece_t[j]] + k_off[j]), &k_lds[buf][(wave + j * TW) * 512]);
+      if (T_UNIFORM) copy_to_lds(kbase[piece_t[j]], k_off[j] * 2, &k_lds[buf][(wave + j * TW) * 512]);
+      else copy_to_lds(kbase[piece_t[j]] + k_off[j], &k_lds[buf][(wave + j * TW) * 512]);
     }
 #pragma unroll
     for (int j = 0; j < TPT; ++j) {
       if (TCH % (TW * 64) != 0 && wave * 64 + j * (TW * 64) >= TCH) break;
-      if (T_UNIFORM) copy_to_lds(plane + vbase[piece_t[j]], v_off[j] * 2, &v_lds[buf][(wave + j * TW) * 512]);
-      else copy_to_lds(plane + (vbase[piece_t[j]] + v_off[j]), &v_lds[buf][(wave + j * TW) * 512]);
+      if (T_UNIFORM) copy_to_lds(vbase[piece_t[j]], v_off[j] * 2, &v_lds[buf][(wave + j * TW) * 512]);
+      else copy_to_lds(vbase[piece_t[j]] + v_off[j], &v_lds[buf][(wave + j * TW) * 512]);
     }
   };
   // the copies this wave has issued are in LDS
@@ -556,11 +586,10 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
           st[t][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[dc], qb[nb][dc], st[t][nb], 0, 0, 0);
     }
   };
-  // a step's scores without the keys that a column may not see; a step inside every column's range needs none of it
+  // a step's scores without the keys that a column may not see (steps outside `free` only)
   auto mask = [&](int s, f32x4 (&st)[2][NB]) {
     const int kb = k_lo + s * 32;
     const bool ok0 = kb < k_hi, ok1 = kb + 16 < k_hi;
-    if (ok0 && ok1 && kb + 31 <= p_first && kb >= lo_last) return;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -572,63 +601,51 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
           st[t][nb][i] = ok ? st[t][nb][i] : -INFINITY;
         }
   };
-  // running maximum and sum per column, P in bfloat16 as the B operand of the second product
-  auto softmax = [&](const f32x4 (&st)[2][NB], bf16x8 (&pb)[NB], float (&alpha)[NB]) -> bool {
-    bool grew = false;
+  // The running maximum of a column follows its scores in jumps: it moves only when a score exceeds it by more than
+  // 2^8, so that weights stay below 2^8 and, on most steps, nothing moves. Whether anything does is asked of every
+  // lane's own scores first; only then are the maxima of the four key groups brought together, the sums and the
+  // output so far scaled down (alpha is exactly 1 for a column that stays).
+  auto follow_maximum = [&](const f32x4 (&st)[2][NB]) {
+    float tmax[NB];
+    bool over = false;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-      float sc[8];
-      float tmax = -INFINITY;
+      tmax[nb] = max3(max3(st[0][nb][0], st[0][nb][1], st[0][nb][2]), max3(st[0][nb][3], st[1][nb][0], st[1][nb][1]),
+                      max3(st[1][nb][2], st[1][nb][3], st[1][nb][3]));
+      over = over || tmax[nb] * scale_log2 > m[nb] + 8.f;
+    }
+    if (__builtin_amdgcn_ballot_w64(over) == 0) return;
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+    for (int nb = 0; nb < NB; ++nb) {
+      const float top = column_max(tmax[nb]) * scale_log2;
+      const float m_new = top > m[nb] + 8.f ? top : m[nb];
+      const float alpha = __builtin_amdgcn_exp2f(m[nb] - m_new);
+      m[nb] = m_new;
+      l[nb] *= alpha;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float v = st[t][nb][i];
-          sc[t * 4 + i] = v;
-          tmax = fmaxf(tmax, v);
-        }
-      tmax = column_max(tmax) * scale_log2;
-      // the exponent follows the running maximum in jumps, as in the wave kernel
-      const bool move = tmax > m[nb] + 8.f || m[nb] == -INFINITY;
-      const float m_new = move ? fmaxf(m[nb], tmax) : m[nb];
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      grew = grew || (move && m_new > m[nb]);
-      alpha[nb] = __builtin_amdgcn_exp2f(m[nb] - m_use);
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[nb][db][i] *= alpha;
+    }
+  };
+  // the weights of a step's keys: P in bfloat16 as the B operand of the second product, their sums in 32-bit
+  auto weights = [&](const f32x4 (&st)[2][NB], bf16x8 (&pb)[NB]) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
       float psum = 0.f;
       bf16x8 pv;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = __builtin_amdgcn_exp2f(fmaf(sc[e], scale_log2, -m_use));
+        const float p = __builtin_amdgcn_exp2f(fmaf(st[e >> 2][nb][e & 3], scale_log2, -m[nb]));
         psum += p;
         pv[e] = static_cast<__bf16>(p);
       }
       pb[nb] = pv;
-      l[nb] = l[nb] * alpha[nb] + psum;
-      m[nb] = m_new;
+      l[nb] += psum;
     }
-    return __builtin_amdgcn_ballot_w64(grew) != 0;
   };
-  // O^T = O^T * alpha + V^T . P^T; while no column of the wave has a new maximum every alpha is exactly 1.
-  // EDGE: the step holds keys that no row of the tile may see (past its last position, before its first window,
-  // past its last page). Their weights are zero, but their values are whatever an earlier owner of the page left,
-  // possibly not even finite: they are replaced by zeros before the product.
-  auto values = [&](int s, int buf, const bf16x8 (&pb)[NB], const float (&alpha)[NB], bool rescale, const bool EDGE) {
-    if (rescale) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) o[nb][db][i] *= alpha[nb];
-    }
-    bool dead[8];
-    if (EDGE) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int key = k_lo + s * 32 + (e >> 2) * 16 + g * 4 + (e & 3);
-        dead[e] = !(key <= tp_last && key >= t_lo);
-      }
-    }
+  // O^T += V^T . P^T
+  auto values = [&](int buf, const bf16x8 (&pb)[NB]) {
     constexpr int HALF = (DB + 1) / 2;      // the head in two halves: as many operands in registers at a time
 #pragma unroll
     for (int h = 0; h < DB; h += HALF) {
@@ -638,11 +655,6 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
         const bf16* vp = &v_lds[buf][((db * 2 + (g >> 1)) * 16 + c16) * 8 + (g & 1) * 4];
         const bf16x4 h0 = load4(vp), h1 = load4(vp + DB * 256);
         va[db - h] = (bf16x8){h0[0], h0[1], h0[2], h0[3], h1[0], h1[1], h1[2], h1[3]};
-        if (EDGE) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (dead[e]) va[db - h][e] = static_cast<__bf16>(0.f);
-        }
       }
 #pragma unroll
       for (int db = h; db < h + HALF && db < DB; ++db)
@@ -651,45 +663,65 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
           o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[db - h], pb[nb], o[nb][db], 0, 0, 0);
     }
   };
-  // inside: every key of step s is one that some row of the tile sees
-  auto inside = [&](int s) { return k_lo + s * 32 + 31 <= tp_last && k_lo + s * 32 >= t_lo; };
-  // a wave skips the steps whose keys all lie past its last row or before its first window
-  auto mine = [&](int s) { return active && s < s_end && k_lo + s * 32 <= p_last && k_lo + s * 32 + 31 >= w_lo; };
+  // A step outside `inside` holds keys that no row of the tile may see (past its last position, before its first
+  // window, past its last page). Their weights are zero, but their values are whatever an earlier owner of the page
+  // left, possibly not even finite, and zero times that is no number. Such a step's values are therefore set to zero
+  // in LDS, a turn before any wave multiplies by them: wave w takes the 8 keys w*8.. of the step, a lane a piece
+  // (8 keys of one element of the head) at a time. The barrier that ends the turn publishes it.
+  auto zero_unseen_values = [&](int s, int buf) {
+    const int key0 = k_lo + s * 32 + wave * 8;
+    if (key0 >= t_lo && key0 + 7 <= tp_last) return;
+    for (int piece = lane; piece < 16 * DB; piece += 64) {
+      bf16* vp = &v_lds[buf][((((wave >> 1) * DB + (piece >> 4)) * 2 + (wave & 1)) * 16 + (piece & 15)) * 8];
+      bf16x8 v = load8(vp);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (key0 + e < t_lo || key0 + e > tp_last) v[e] = static_cast<__bf16>(0.f);
+      *reinterpret_cast<bf16x8*>(vp) = v;
+    }
+  };
+  auto mine = [&](int s) { return s >= mine_lo && s < mine_hi; };
 
   if (s_begin < s_end) {
-    // Steps s_begin and s_begin + 1 go to LDS before the loop; the loop's turn s copies step s + 2, multiplies out
-    // the scores of step s + 1 and finishes step s. Buffer of step s: (s - s_begin) % TBUF.
+    // Steps s_begin and s_begin + 1 go to LDS before the loop; turn s copies step s + 2, multiplies out the scores of
+    // step s + 1 (into `ahead`) and finishes step s (from `now`). Buffer of step s: (s - s_begin) % TBUF.
     load_run(s_begin);
     stage(s_begin, 0);
     if (s_begin + 1 < s_end) stage(s_begin + 1, 1);
     staged();
     __syncthreads();
-    f32x4 st_cur[2][NB], st_next[2][NB];
-    if (mine(s_begin)) {
-      scores(0, st_cur);
-      mask(s_begin, st_cur);
+    if (s_begin < in_lo || s_begin >= in_hi) {     // the same for all waves
+      zero_unseen_values(s_begin, 0);
+      __syncthreads();
     }
-    int buf = 0;                                   // of step s
-    for (int s = s_begin; s < s_end; ++s) {
+    f32x4 st_even[2][NB], st_odd[2][NB];
+    scores(0, st_even);
+    if (s_begin < free_lo || s_begin >= free_hi) mask(s_begin, st_even);
+    // The scores of the step ahead are multiplied out whether or not this wave will use them (a wave skips few
+    // steps, and after the split's last step they are thrown away): so they are defined on every path, and the
+    // compiler keeps them where they are instead of copying them about.
+    auto turn = [&](int s, int buf, f32x4 (&now)[2][NB], f32x4 (&ahead)[2][NB]) {
       const int buf1 = buf + 1 == TBUF ? 0 : buf + 1, buf2 = buf1 + 1 == TBUF ? 0 : buf1 + 1;
       if (s + 2 < s_end) stage(s + 2, buf2);
-      const bool cur = mine(s), next = mine(s + 1);
-      bf16x8 pb[NB];
-      float alpha[NB];
-      if (next) scores(buf1, st_next);
-      if (cur) {
-        const bool rescale = softmax(st_cur, pb, alpha);
-        values(s, buf, pb, alpha, rescale, !inside(s));
+      scores(buf1, ahead);
+      if (mine(s)) {
+        bf16x8 pb[NB];
+        follow_maximum(now);
+        weights(now, pb);
+        values(buf, pb);
       }
-      if (next) mask(s + 1, st_next);
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) st_cur[t][nb] = st_next[t][nb];
-      buf = buf1;
+      if (s + 1 < free_lo || s + 1 >= free_hi) mask(s + 1, ahead);
+      if ((s + 1 < in_lo || s + 1 >= in_hi) && s + 1 < s_end) zero_unseen_values(s + 1, buf1);
       // everyone has read step s's buffer (the copy of step s + 3 overwrites it) and step s + 2 has arrived
       staged();
       __syncthreads();
+      return buf1;
+    };
+    int buf = 0;                                   // of step s
+    for (int s = s_begin; s < s_end; s += 2) {     // two turns a round: the scores change places without being moved
+      buf = turn(s, buf, st_even, st_odd);
+      if (s + 1 >= s_end) break;
+      buf = turn(s + 1, buf, st_odd, st_even);
     }
   }
 
@@ -712,7 +744,7 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
       float* dst = part_o + slot * HD + g * 4;
 #pragma unroll
       for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + db * 16) = o[nb][db];
-      if (g == 0) part_ml[slot] = make_float2(m[nb], lt);
+      if (g == 0) part_ml[slot] = make_float2(m[nb] == NO_MAX ? -INFINITY : m[nb], lt);
     }
   }
 }

@@ -369,23 +369,35 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
 // ---- Long portions of prompts: a workgroup of four waves shares every step's keys and values through LDS ----
 //
 // A wave of the kernel above fetches its keys and values itself, so the rows of a prompt read each key once per
-// 16*NB columns, and a wave waits out the fetch of every step. Here a *tile* is up to TW * (16 * TNB / group size)
-// consecutive rows of one request; its four waves own 16 * TNB columns each and walk the tile's keys together. Each
-// step's 32 keys and values are copied once from the pages into LDS, two steps ahead of the products that read
-// them, by loads that write LDS directly (global_load_lds: no registers, no store instructions), and every wave takes
-// its operands from there. LDS holds them in the order the products read them: 16-byte pieces, the 64 pieces of one
-// operand fetch side by side, so that reads meet no bank conflict and need no padding; a copying lane picks the
-// piece of the page that belongs in its slot. The arithmetic of a step is the wave kernel's, in another order: the
-// scores of step s+1 are multiplied out (matrix cores) while the exponentials of step s are taken (vector unit), so
-// that a wave keeps both busy. (Heads wider than 128: 16 columns a wave.)
+// 16*NB columns, and a wave waits out the fetch of every step. Here a *tile* is up to TW * (32 / group size)
+// consecutive rows of one request; its four waves own 32 columns each, one a lane pair, and walk the tile's keys
+// together. Each step's 32 keys and values are copied once from the pages into LDS, two steps ahead of the products
+// that read them, by loads that write LDS directly (global_load_lds: no registers, no store instructions), and every
+// wave takes its operands from there. LDS holds them in the order the products read them: 16-byte pieces, 16 pieces
+// that a quarter of a wave reads together side by side, so that reads meet no bank conflict and need no padding; a
+// copying lane picks the piece of the page that belongs in its slot.
+//
+// Both products are v_mfma_f32_32x32x16_bf16, with the column on the lane as in the wave kernel:
+//   S^T[32 keys, 32 columns] = K . Q^T over the head in steps of 16; lane (c, h) of the result holds column c and the
+//       score rows 8b + 4h + k (b, k < 4) in accumulator 4b + k
+//   O^T[32 of the head, 32 columns] += V^T . P^T over the keys in two halves of 16; as the second operand lane (c, h)
+//       must hold P of the keys 8h .. 8h+7 of a half
+// So that P can stay in the registers S^T left it in, score row 8b + 4h + k is made to be key 16 (b >> 1) + 8h +
+// 4 (b & 1) + k: inside each 16-key tile the rows' bits 2 and 3 change places, which costs nothing, since the copying
+// lane picks its key anyway. Accumulators 0..7 of a lane are then the keys 8h.. of the first half and 8..15 those of
+// the second, in order.
 static constexpr int TW = 4;               // waves of a tile
-static constexpr int TNB = HD > 128 ? 1 : 2;   // column blocks of a wave: what leaves registers for several waves a SIMD
+static constexpr int TCOLS = 32;           // columns of a wave
 static constexpr int TBUF = 3;             // LDS buffers: step s+1's keys, step s's values, and step s+2 being written
 static constexpr int NCH = HD / 8;         // 16-byte pieces of one key
 static constexpr int TCH = 4 * HD;         // pieces of a step's keys, and of its values: HD / 16 fetches of 64
 static constexpr int TPT = (TCH + TW * 64 - 1) / (TW * 64);   // fetches a wave issues, of each
-// keys:   piece (t, dch, c16) = key t*16 + c16, elements dch*8.. at piece index (t*NCH + dch)*16 + c16
+static constexpr int KC = HD / 16;         // 16-wide steps of the head for K.Q
+static constexpr int DT = (HD + 31) / 32;  // 32-high blocks of the head for V.P
+// keys:   piece (t, dch, r) = key t*16 + (r with bits 2 and 3 exchanged), elements dch*8.. at piece index
+//         (t*NCH + dch)*16 + r
 // values: piece (t, db, gh, c16) = element db*16 + c16 of the head, keys t*16 + gh*8.. at ((t*DB + db)*2 + gh)*16 + c16
+typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 #pragma clang diagnostic ignored "-Winline-asm"   // M0 in a clobber list: meant
 // One 16-byte piece per lane from global memory straight into LDS: lane i's piece lands at lds_base + 16 * i
@@ -404,55 +416,56 @@ __device__ __forceinline__ void copy_to_lds(const bf16* src, unsigned lane_bytes
                           (unsigned)__builtin_amdgcn_readfirstlane((int)a);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_bytes), "s"(scalar), "s"(base) : "memory", "m0");
 }
+// the larger / the sum of a value on the two lanes that hold one column of a tile (they differ in lane bit 5)
+__device__ __forceinline__ float pair_max(float v) {
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float pair_sum(float v) {
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
 
+// (heads wider than 128 need more than 256 registers a lane: one wave a SIMD)
 template <bool PS16>
-__global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) void attention_tile_kernel(
+__global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1))) void attention_tile_kernel(
     const bf16* __restrict__ q, long q_ld, const bf16* __restrict__ plane, const int* __restrict__ block_tables,
     int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ tiles,
     bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
     int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits, int max_steps,
     int split_stride, int* __restrict__ row_splits) {
-  constexpr int NB = TNB;
   __shared__ __attribute__((aligned(16))) bf16 k_lds[TBUF][TCH * 8];
   __shared__ __attribute__((aligned(16))) bf16 v_lds[TBUF][TCH * 8];
   const int page_size = PS16 ? 16 : page_size_arg;
   const int tile = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   // the wave's number is the same on all its lanes: said so, what follows from it is scalar arithmetic and branches
-  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c16 = lane & 15, g = lane >> 4;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c32 = lane & 31, h = lane >> 5;
   const int t_row0 = tiles[tile].x, t_rows = tiles[tile].y;
   const int* bt = block_tables + (long)row_seq[t_row0] * bt_ld;
   const int tp_first = positions[t_row0], tp_last = tp_first + t_rows - 1;
 
   // the wave's rows of the tile; a wave past the tile's last row only helps with the copies
-  const int rows_per_wave = (16 * NB) / group_size;
+  const int rows_per_wave = TCOLS / group_size;
   const int n_rows = max(0, min(rows_per_wave, t_rows - wave * rows_per_wave));
   const bool active = n_rows > 0;
   const int row0 = t_row0 + (active ? wave * rows_per_wave : 0);
   const int p_first = tp_first + (active ? wave * rows_per_wave : 0);
   const int p_last = p_first + n_rows - 1;
 
-  int col_row[NB], col_head[NB], col_pos[NB], col_lo[NB];
-  bool col_ok[NB];
+  // the lane's column: a row of the wave and a query head of the group
+  const int ro = c32 / group_size;
+  const bool col_ok = ro < n_rows;
+  const int col_row = row0 + (col_ok ? ro : 0);
+  const int col_head = kvh * group_size + c32 % group_size;
+  const int col_pos = col_ok ? p_first + ro : -1;
+  const int col_lo = (window > 0 && col_pos - window + 1 > 0) ? col_pos - window + 1 : 0;
+  bf16x8 qb[KC];
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int c = nb * 16 + c16;
-    const int ro = c / group_size;
-    col_ok[nb] = ro < n_rows;
-    col_row[nb] = row0 + (col_ok[nb] ? ro : 0);
-    col_head[nb] = kvh * group_size + c % group_size;
-    col_pos[nb] = col_ok[nb] ? p_first + ro : -1;
-    col_lo[nb] = (window > 0 && col_pos[nb] - window + 1 > 0) ? col_pos[nb] - window + 1 : 0;
+  for (int kc = 0; kc < KC; ++kc) {
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (col_ok) v = load8(q + (long)col_row * q_ld + (long)col_head * HD + kc * 16 + h * 8);
+    qb[kc] = v;
   }
-  bf16x8 qb[NB][DC];
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-    for (int dc = 0; dc < DC; ++dc) {
-      const int d = dc * 32 + g * 8;
-      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (col_ok[nb] && d < HD) v = load8(q + (long)col_row[nb] * q_ld + (long)col_head[nb] * HD + d);
-      qb[nb][dc] = v;
-    }
 
   // the tile's keys and this workgroup's share of them, as in the wave kernel
   const int t_lo = (window > 0 && tp_first - window + 1 > 0) ? tp_first - window + 1 : 0;   // first key any row sees
@@ -474,17 +487,16 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   const long v_head = ((long)n_kv_heads + kvh) * page_size * HD;
 
   // No running maximum yet: a finite number far below any score, so that differences with it stay numbers (a
-  // column none of whose keys has counted so far keeps it, with a sum of zero; the merge gives such a part no weight)
+  // column none of whose keys has counted so far keeps it, with a sum of zero; the merge gives such a part no weight).
+  // `over`: the raw score from which on the maximum has to move.
   constexpr float NO_MAX = -1e30f;
-  f32x4 o[NB][DB];
-  float m[NB], l[NB];
+  const float per_scale = 1.f / scale_log2;
+  f32x16 o[DT];
+  float m = NO_MAX, l = 0.f, over = (NO_MAX + 8.f) * per_scale;
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    m[nb] = NO_MAX;
-    l[nb] = 0.f;
+  for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int db = 0; db < DB; ++db) o[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  }
+    for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
 
   // What the loop below spends per step is instructions, of any kind: a wave issues one every four cycles at best,
   // and the matrix instructions of the other wave on its SIMD do not hide the rest. So whatever a step can know in
@@ -492,7 +504,7 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   //   mine:   steps with a key that some row of this wave sees (others are skipped: past its last row, before its
   //           first window)
   //   free:   steps all of whose keys every row of the wave sees (no masking)
-  //   inside: steps all of whose keys some row of the tile sees (their values need no guarding, see `values`)
+  //   inside: steps all of whose keys some row of the tile sees (their values need no guarding, see below)
   const int mine_lo = max(s_begin, (w_lo - k_lo) >> 5), mine_hi = active ? min(s_end, ((p_last - k_lo) >> 5) + 1) : 0;
   const int free_lo = (lo_last - k_lo + 31) >> 5, free_hi = (p_first + 1 - k_lo) >> 5;
   const int in_lo = (t_lo - k_lo + 31) >> 5, in_hi = (tp_last + 1 - k_lo) >> 5;
@@ -526,7 +538,8 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     const int c = tid + j * (TW * 64);                      // the piece's index in LDS
     const int t = c / (2 * HD);                             // keys and values alike
     piece_t[j] = T_IS_J ? j : T_UNIFORM ? __builtin_amdgcn_readfirstlane(t) : t;
-    k_off[j] = (unsigned)k_head + (c & 15) * HD + ((c >> 4) % NCH) * 8;
+    const int key_in_tile = (c & 3) | ((c & 4) << 1) | ((c & 8) >> 1);
+    k_off[j] = (unsigned)k_head + key_in_tile * HD + ((c >> 4) % NCH) * 8;
     v_off[j] = (unsigned)v_head + (((c >> 5) % DB) * 16 + (c & 15)) * page_size + ((c >> 4) & 1) * 8;
   }
 
@@ -564,103 +577,70 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   // the copies this wave has issued are in LDS
   auto staged = [&]() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); };
 
-  // S^T of one step, one 16-key tile after the other (its keys are asked for together), dc by dc over the column
-  // blocks' independent sums
-  auto scores = [&](int buf, f32x4 (&st)[2][NB]) {
+  // S^T of one step. Lane (c, h) supplies score row c (tile c >> 4, row c & 15 of it), elements kc*16 + h*8.. of the head.
+  auto scores = [&](int buf, f32x16& st) {
+    const bf16* kp = &k_lds[buf][(((c32 >> 4) * NCH + h) * 16 + (c32 & 15)) * 8];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      bf16x8 ka[DC];
+    for (int i = 0; i < 16; ++i) st[i] = 0.f;
 #pragma unroll
-      for (int dc = 0; dc < DC; ++dc) {
-        const int d = dc * 32 + g * 8;
-        const bool d_ok = (HD % 32 == 0) || d < HD;
-        ka[dc] = load8(&k_lds[buf][(((t * NCH + (d_ok ? dc * 4 + g : 0)) * 16) + c16) * 8]);
-        if (!d_ok) ka[dc] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-      }
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) st[t][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int dc = 0; dc < DC; ++dc)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          st[t][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[dc], qb[nb][dc], st[t][nb], 0, 0, 0);
-    }
+    for (int kc = 0; kc < KC; ++kc)
+      st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load8(kp + kc * 256), qb[kc], st, 0, 0, 0);
   };
-  // a step's scores without the keys that a column may not see (steps outside `free` only)
-  auto mask = [&](int s, f32x4 (&st)[2][NB]) {
-    const int kb = k_lo + s * 32;
-    const bool ok0 = kb < k_hi, ok1 = kb + 16 < k_hi;
+  // a step's scores without the keys that the column may not see (steps outside `free` only); accumulator i of
+  // lane (c, h) is key 16 (i >> 3) + 8h + (i & 7) of the step
+  auto mask = [&](int s, f32x16& st) {
+    asm volatile("; a step with masked keys");   // (keeps the compiler from doing this on every step, by selects)
+    const int kb = k_lo + s * 32 + h * 8;
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = kb + t * 16 + g * 4 + i;
-          const bool ok = (t ? ok1 : ok0) && key <= col_pos[nb] && key >= col_lo[nb];
-          st[t][nb][i] = ok ? st[t][nb][i] : -INFINITY;
-        }
+    for (int i = 0; i < 16; ++i) {
+      const int key = kb + (i >> 3) * 16 + (i & 7);
+      st[i] = (key <= col_pos && key >= col_lo) ? st[i] : -INFINITY;
+    }
   };
   // The running maximum of a column follows its scores in jumps: it moves only when a score exceeds it by more than
   // 2^8, so that weights stay below 2^8 and, on most steps, nothing moves. Whether anything does is asked of every
-  // lane's own scores first; only then are the maxima of the four key groups brought together, the sums and the
+  // lane's own scores first; only then are the maxima of a column's two lanes brought together, the sum and the
   // output so far scaled down (alpha is exactly 1 for a column that stays).
-  auto follow_maximum = [&](const f32x4 (&st)[2][NB]) {
-    float tmax[NB];
-    bool over = false;
+  auto follow_maximum = [&](const f32x16& st) {
+    const float tmax = max3(max3(max3(st[0], st[1], st[2]), max3(st[3], st[4], st[5]), max3(st[6], st[7], st[8])),
+                            max3(st[9], st[10], st[11]), max3(max3(st[12], st[13], st[14]), st[15], st[15]));
+    if (__builtin_amdgcn_ballot_w64(tmax > over) == 0) return;
+    const float top = pair_max(tmax) * scale_log2;
+    const float m_new = top > m + 8.f ? top : m;
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+    m = m_new;
+    over = (m_new + 8.f) * per_scale;
+    l *= alpha;
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      tmax[nb] = max3(max3(st[0][nb][0], st[0][nb][1], st[0][nb][2]), max3(st[0][nb][3], st[1][nb][0], st[1][nb][1]),
-                      max3(st[1][nb][2], st[1][nb][3], st[1][nb][3]));
-      over = over || tmax[nb] * scale_log2 > m[nb] + 8.f;
-    }
-    if (__builtin_amdgcn_ballot_w64(over) == 0) return;
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      const float top = column_max(tmax[nb]) * scale_log2;
-      const float m_new = top > m[nb] + 8.f ? top : m[nb];
-      const float alpha = __builtin_amdgcn_exp2f(m[nb] - m_new);
-      m[nb] = m_new;
-      l[nb] *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[nb][db][i] *= alpha;
-    }
+      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
   };
-  // the weights of a step's keys: P in bfloat16 as the B operand of the second product, their sums in 32-bit
-  auto weights = [&](const f32x4 (&st)[2][NB], bf16x8 (&pb)[NB]) {
+  // the weights of a step's keys: P in bfloat16 as the second operand of V.P, one for each half of the keys, and their
+  // sum in 32-bit
+  auto weights = [&](const f32x16& st, bf16x8 (&pb)[2]) {
+    float psum = 0.f;
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      float psum = 0.f;
-      bf16x8 pv;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float p = __builtin_amdgcn_exp2f(fmaf(st[e >> 2][nb][e & 3], scale_log2, -m[nb]));
-        psum += p;
-        pv[e] = static_cast<__bf16>(p);
-      }
-      pb[nb] = pv;
-      l[nb] += psum;
+    for (int i = 0; i < 16; ++i) {
+      const float p = __builtin_amdgcn_exp2f(fmaf(st[i], scale_log2, -m));
+      psum += p;
+      pb[i >> 3][i & 7] = static_cast<__bf16>(p);
     }
+    l += psum;
   };
-  // O^T += V^T . P^T
-  auto values = [&](int buf, const bf16x8 (&pb)[NB]) {
-    constexpr int HALF = (DB + 1) / 2;      // the head in two halves: as many operands in registers at a time
+  // O^T += V^T . P^T. Lane (c, h) supplies element dt*32 + c of the head, keys 8h.. of each half.
+  auto values = [&](int buf, const bf16x8 (&pb)[2]) {
 #pragma unroll
-    for (int h = 0; h < DB; h += HALF) {
-      bf16x8 va[HALF];
+    for (int dt = 0; dt < DT; ++dt) {
+      const int db = 2 * dt + (c32 >> 4);
+      const bool d_ok = (HD % 32 == 0) || db < DB;
+      const bf16* vp = &v_lds[buf][(((d_ok ? db : 0) * 2 + h) * 16 + (c32 & 15)) * 8];
 #pragma unroll
-      for (int db = h; db < h + HALF && db < DB; ++db) {
-        const bf16* vp = &v_lds[buf][((db * 2 + (g >> 1)) * 16 + c16) * 8 + (g & 1) * 4];
-        const bf16x4 h0 = load4(vp), h1 = load4(vp + DB * 256);
-        va[db - h] = (bf16x8){h0[0], h0[1], h0[2], h0[3], h1[0], h1[1], h1[2], h1[3]};
+      for (int half = 0; half < 2; ++half) {
+        bf16x8 va = load8(vp + half * DB * 256);
+        if (!d_ok) va = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[half], o[dt], 0, 0, 0);
       }
-#pragma unroll
-      for (int db = h; db < h + HALF && db < DB; ++db)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          o[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[db - h], pb[nb], o[nb][db], 0, 0, 0);
     }
   };
   // A step outside `inside` holds keys that no row of the tile may see (past its last position, before its first
@@ -694,22 +674,20 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
       zero_unseen_values(s_begin, 0);
       __syncthreads();
     }
-    f32x4 st_even[2][NB], st_odd[2][NB];
+    f32x16 st_even, st_odd;
     scores(0, st_even);
     if (s_begin < free_lo || s_begin >= free_hi) mask(s_begin, st_even);
     // The scores of the step ahead are multiplied out whether or not this wave will use them (a wave skips few
     // steps, and after the split's last step they are thrown away): so they are defined on every path, and the
     // compiler keeps them where they are instead of copying them about.
-    auto turn = [&](int s, int buf, f32x4 (&now)[2][NB], f32x4 (&ahead)[2][NB]) {
+    auto turn = [&](int s, int buf, f32x16& now, f32x16& ahead) {
       const int buf1 = buf + 1 == TBUF ? 0 : buf + 1, buf2 = buf1 + 1 == TBUF ? 0 : buf1 + 1;
       if (s + 2 < s_end) stage(s + 2, buf2);
+      bf16x8 pb[2];
       scores(buf1, ahead);
-      if (mine(s)) {
-        bf16x8 pb[NB];
-        follow_maximum(now);
-        weights(now, pb);
-        values(buf, pb);
-      }
+      follow_maximum(now);
+      weights(now, pb);
+      values(buf, pb);
       if (s + 1 < free_lo || s + 1 >= free_hi) mask(s + 1, ahead);
       if ((s + 1 < in_lo || s + 1 >= in_hi) && s + 1 < s_end) zero_unseen_values(s + 1, buf1);
       // everyone has read step s's buffer (the copy of step s + 3 overwrites it) and step s + 2 has arrived
@@ -725,27 +703,33 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     }
   }
 
+  // accumulator 4b + k of lane (c, h) and block dt is element dt*32 + 8b + 4h + k of the head
+  const float lt = pair_sum(l);
+  if (!col_ok) return;
+  if (item_splits == 1) {
+    const float inv = 1.f / lt;
+    bf16* dst = out + (long)col_row * out_ld + (long)col_head * HD + h * 4;
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const float lt = column_sum(l[nb]);
-    if (!col_ok[nb]) continue;
-    if (item_splits == 1) {
-      const float inv = 1.f / lt;
-      bf16* dst = out + (long)col_row[nb] * out_ld + (long)col_head[nb] * HD + g * 4;
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
+      for (int b = 0; b < 4; ++b) {
+        if (HD % 32 != 0 && dt * 32 + b * 8 >= HD) continue;
         bf16x4 w;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) w[i] = static_cast<__bf16>(o[nb][db][i] * inv);
-        *reinterpret_cast<bf16x4*>(dst + db * 16) = w;
+        for (int k = 0; k < 4; ++k) w[k] = static_cast<__bf16>(o[dt][b * 4 + k] * inv);
+        *reinterpret_cast<bf16x4*>(dst + dt * 32 + b * 8) = w;
       }
-    } else {
-      const long slot = ((long)col_row[nb] * n_heads + col_head[nb]) * split_stride + split;
-      float* dst = part_o + slot * HD + g * 4;
+  } else {
+    const long slot = ((long)col_row * n_heads + col_head) * split_stride + split;
+    float* dst = part_o + slot * HD + h * 4;
 #pragma unroll
-      for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + db * 16) = o[nb][db];
-      if (g == 0) part_ml[slot] = make_float2(m[nb] == NO_MAX ? -INFINITY : m[nb], lt);
-    }
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        if (HD % 32 != 0 && dt * 32 + b * 8 >= HD) continue;
+        *reinterpret_cast<f32x4*>(dst + dt * 32 + b * 8) = (f32x4){o[dt][b * 4], o[dt][b * 4 + 1], o[dt][b * 4 + 2], o[dt][b * 4 + 3]};
+      }
+    if (h == 0) part_ml[slot] = make_float2(m == NO_MAX ? -INFINITY : m, lt);
   }
 }
 
@@ -877,7 +861,7 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_rows_kernel(const flo
 
 TIS_EXPORT int tis_attention_mfma_head_dim() { return HD; }
 // columns (row, query head of a group) that one wave of a tile holds; a tile has four waves
-TIS_EXPORT int tis_attention_mfma_tile_columns() { return 16 * TNB; }
+TIS_EXPORT int tis_attention_mfma_tile_columns() { return TCOLS; }
 
 // items: (first row, rows) pairs; the rows of an item are consecutive positions of one request and
 // rows * group_size <= 16 * nb. Null: n_items single rows, item i being row i. tiles: (first row, rows) pairs for the
@@ -945,7 +929,7 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
   } else {
     n_splits = 1;
   }
-  if (n_tiles > 0 && group > 16 * TNB) return tis_fail("attention_mfma: a group of %d query heads does not fit a tile's wave", group);
+  if (n_tiles > 0 && group > TCOLS) return tis_fail("attention_mfma: a group of %d query heads does not fit a tile's wave", group);
   if (n_tiles > 0 && 4L * n_kv_heads * page_size * HD >= (1L << 31))
     return tis_fail("attention_mfma: a page of %d key/value heads x %d slots is too large for the tile kernel's 32-bit offsets", n_kv_heads, page_size);
   if (n_tiles == 0) tile_splits = 1;

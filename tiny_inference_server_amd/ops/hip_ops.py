@@ -173,7 +173,7 @@ _ATTN_WORKSPACE_FLOATS = 16 << 20
 
 def tile_columns(head_dim: int) -> int:
     """Columns (row, query head of a group) of one wave of the tile kernel, as the kernel source sets them."""
-    return 32 if head_dim <= 128 else 16
+    return 32
 
 
 def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: int = 0):

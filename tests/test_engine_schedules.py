@@ -131,11 +131,11 @@ def test_all_schedules_agree_with_each_other(backend):
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["B", "C", "D"])
 def test_schedules_with_portions_on_the_tile_kernel(name, monkeypatch):
-    """The tiny models' prompts are too little work for the workgroup attention kernel to be chosen; here it is made
-    to take every portion that fills half a tile, and whole prompts, portions and mixed batches (with pages handed
-    out again) are compared with the plain implementation as elsewhere."""
+    """Beside decoded tokens deep in their requests the tiny models' portions are too little work for the workgroup
+    attention kernel to be chosen; here it is made to take every portion that fills half a tile, and whole prompts,
+    portions and mixed batches (with pages handed out again) are compared with the plain implementation as elsewhere."""
     from tiny_inference_server_amd.ops import hip_ops
-    monkeypatch.setattr(hip_ops, "_ATTN_TILE_MIN_WORK", 0)
+    monkeypatch.setattr(hip_ops, "_ATTN_TILE_MIN_WORK_MIXED", 0)
     planned = {"tiles": 0}
     plan = hip_ops.attention_items
 

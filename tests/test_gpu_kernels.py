@@ -290,12 +290,18 @@ def test_mixed_rows_with_key_splits_chosen_item_by_item(ops_for, n_heads, n_kv, 
 @pytest.mark.parametrize("n_heads,n_kv,hd,page_size,window", [
     (12, 3, 128, 16, 0), (12, 3, 128, 16, 100), (4, 4, 64, 16, 0), (6, 2, 48, 32, 0), (16, 2, 32, 48, 45),
     (2, 1, 256, 16, 0), (5, 1, 16, 16, 33), (20, 1, 32, 16, 0)])
-def test_long_portions_by_tiles(ops_for, n_heads, n_kv, hd, page_size, window):
+@pytest.mark.parametrize("splits", [False, True])
+def test_long_portions_by_tiles(ops_for, monkeypatch, n_heads, n_kv, hd, page_size, window, splits):
     """Portions long enough for the workgroup kernel (tiles of rows whose four waves share each step's keys through
     LDS), beside rows that stay with the one-wave kernel: a whole prompt that ends mid-tile and mid-page, a portion
-    deep into a long request (its tiles are cut into key splits and merged), a decoded token and a three-row portion.
-    Group sizes that divide a wave's 64 columns and ones that do not; heads wider than 128 have 32-column waves."""
+    deep into a long request, a decoded token and a three-row portion. Once as planned (chains this short are not
+    cut), once with the tiles cut into key splits and merged, as those of long prompts are. Group sizes that divide a
+    wave's 32 columns and ones that do not, head sizes in steps of 16 and of 32."""
+    from tiny_inference_server_amd.ops import hip_ops
     from tiny_inference_server_amd.ops.hip_ops import attention_items, tile_columns
+    if splits:
+        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_FROM", 4)
+        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_SHARE", 1.0)
     ops = ops_for(torch.bfloat16)
     group = n_heads // n_kv
     tile_rows = 4 * (tile_columns(hd) // group)
@@ -324,9 +330,15 @@ def test_long_portions_by_tiles(ops_for, n_heads, n_kv, hd, page_size, window):
         torch.testing.assert_close(got[r].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
 
 
-def test_a_tile_sees_a_far_key_and_a_rows_own_key(ops_for):
-    """Two scores are made to stand out in a long portion: a key far back (in an early split of the tile's keys) for
-    one row, and for another row the key at its own position, the last one the causal mask lets through."""
+@pytest.mark.parametrize("splits", [False, True])
+def test_a_tile_sees_a_far_key_and_a_rows_own_key(ops_for, monkeypatch, splits):
+    """Two scores are made to stand out in a long portion: a key far back (in an early split of the tile's keys, when
+    they are cut) for one row, and for another row the key at its own position, the last one the causal mask lets
+    through."""
+    from tiny_inference_server_amd.ops import hip_ops
+    if splits:
+        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_FROM", 4)
+        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_SHARE", 1.0)
     ops = ops_for(torch.bfloat16)
     n_heads, n_kv, hd, page_size, L = 4, 1, 64, 16, 1200
     plane, tables, ks, vs = make_paged([L], n_kv, hd, page_size, torch.bfloat16, seed=38)

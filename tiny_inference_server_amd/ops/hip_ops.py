@@ -164,10 +164,18 @@ _ATTN_TILE_WAVES = 4            # waves of the workgroup that takes a tile of a 
 _ATTN_TILE_GROUPS = 512         # workgroups of the tile kernel that the chip runs side by side
 _ATTN_TILE_MIN_STEPS = 8        # steps of 32 keys below which a tile's split is not worth its merge
 _ATTN_TILE_SPLIT_SLACK = 1.4    # a split may be this much longer than an even share of all steps
+_ATTN_TILE_SPLIT_FROM = 40      # tiles are cut into key splits only if the longest walks at least this many steps ...
+_ATTN_TILE_SPLIT_SHARE = 0.3    # ... and an even share of all steps is at most this fraction of it: a few long chains.
+                                # Otherwise the merge (a launch, and 32-bit partial results written and read) costs
+                                # more than shorter chains save. 12 heads of 128 over 3, us, splits / none / one-wave
+                                # kernel: 4 prompts of 512 tokens 28.8 / 18.8 / 22.8, 8 of 512 40.8 / 25.4 / 33.2, 4 of
+                                # 1,024 50.6 / 39.5 / 57.2, one of 1,024 29.2 / 28.6 / 29.2; but one of 1,536 35.3 /
+                                # 39.9 / 47.7, of 2,048 42.4 / 51.3 / 69.5, 512 tokens behind 3,000 41.5 / 82.5 / 60.0
 _ATTN_TILE_PARTIAL_BYTES = 40 << 20   # partial results (32-bit, per split) beyond which the merge costs more than
                                       # shorter chains save; at least two splits are always allowed
-_ATTN_TILE_MIN_WORK = 3000      # tile steps times key/value heads below which the one-wave kernel is the faster ...
-_ATTN_TILE_MIN_WORK_MIXED = 1500   # ... and beside decoded tokens deep in their requests (their splits are merged anyway)
+_ATTN_TILE_MIN_WORK_MIXED = 1500   # tile steps times key/value heads below which the one-wave kernel is the faster
+                                   # beside decoded tokens deep in their requests (few tiles with long chains: the
+                                   # one-wave kernel spreads them over more waves, and its splits are merged anyway)
 _ATTN_WORKSPACE_FLOATS = 16 << 20
 
 
@@ -186,11 +194,11 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
     An item (one wave) holds consecutive rows of one request, rows * group_size <= 16 * blocks. When no request has
     more than one row the list is simply every row in order, which the kernel knows without being given a list.
     A tile (a workgroup of four waves, `tile_cols` columns each; 0: no tiles) takes up to 4 * (tile_cols // group_size)
-    consecutive rows of a portion that fills at least half of one. Tiles are made only where their steps times
-    `n_kv_heads` (the workgroups' work) reach _ATTN_TILE_MIN_WORK (0: always): a tile's waves walk its keys in
-    lockstep, which pays when there is work for every compute unit and costs on a short prompt. Measured at 12 heads
-    of 128 over 3 (tiles / one-wave kernel, us): 1,536 rows 40 / 48, 1,024 rows 32 / 29, three portions of 700 rows
-    39 / 34; a portion of 512 rows at 1,000 beside 8 decoded tokens 53 / 65, one of 256 rows 41 / 29.
+    consecutive rows of a portion that fills at least half of one. Beside decoded tokens deep in their requests, tiles
+    are made only where their steps times `n_kv_heads` (the workgroups' work; 0: always) reach
+    _ATTN_TILE_MIN_WORK_MIXED. Measured at 12 heads of 128 over 3 (tiles / one-wave kernel, us): one prompt of 256
+    rows 12.1 / 13.3, of 512 rows 17.5 / 22.3, of 1,024 rows 28.6 / 29.2, 8 of 512 rows 25.4 / 33.2; a portion of 512
+    rows at 1,000 beside 8 decoded tokens at 4,095: 54.9 / 64.7, one of 256 rows 40.6 / 30.1, one of 128 35.9 / 23.9.
     """
     none = np.zeros((0, 2), dtype=np.int32)
     single = all(n <= 1 for _, _, n in seq_rows)
@@ -205,7 +213,7 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
         work = sum(int(((p0 + np.minimum(np.arange(0, n, tile_rows) + tile_rows, n) + 31) // 32).sum())
                    for _, p0, n in tiled) * n_kv_heads
         deep = any(n == 1 and p0 >= 512 for _, p0, n in seq_rows)
-        if work < (_ATTN_TILE_MIN_WORK_MIXED if deep else _ATTN_TILE_MIN_WORK):
+        if deep and work < _ATTN_TILE_MIN_WORK_MIXED:
             tiled = []
     taken = {f for f, _, _ in tiled}
     rest = [(f, p0, n) for f, p0, n in seq_rows if n > 0 and f not in taken]
@@ -360,10 +368,11 @@ def attention_launch_plan(n, n_items, n_tiles, tile_steps, single, max_kv_len, n
         # 196 / 260; 4,096 rows: 146 / 202.
         all_steps, longest = tile_steps
         share = all_steps * n_kv_heads / _ATTN_TILE_GROUPS
-        tile_max_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
-        most_splits = max(2, _ATTN_TILE_PARTIAL_BYTES // (n * n_heads * head_dim * 4))
-        tile_splits = max(1, min(most_splits, -(-longest // tile_max_steps)))
-        tile_max_steps = max(tile_max_steps, -(-longest // tile_splits))
+        if longest >= _ATTN_TILE_SPLIT_FROM and share <= _ATTN_TILE_SPLIT_SHARE * longest:
+            tile_max_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
+            most_splits = max(2, _ATTN_TILE_PARTIAL_BYTES // (n * n_heads * head_dim * 4))
+            tile_splits = max(1, min(most_splits, -(-longest // tile_max_steps)))
+            tile_max_steps = max(tile_max_steps, -(-longest // tile_splits))
     # partial results of split key ranges live in one workspace of fixed size; fewer splits where it
     # would not suffice
     most = max(1, (workspace_floats - n) // (n * n_heads * (head_dim + 2)))

@@ -75,7 +75,8 @@ def tile_extents(HD, kvh_count, tiles, positions, lp, table_width):
         for j in range(TPT):
             c = tid + j * TW * 64
             live = (tid // 64) * 64 + j * TW * 64 < TCH          # the kernel's break for pieces past the step's last
-            k_off = k_head + (c & 15) * HD + ((c >> 4) % NCH) * 8
+            key_in_tile = (c & 3) | ((c & 4) << 1) | ((c & 8) >> 1)
+            k_off = k_head + key_in_tile * HD + ((c >> 4) % NCH) * 8
             v_off = v_head + (((c >> 5) % DB) * 16 + (c & 15)) * PAGE + ((c >> 4) & 1) * 8
             worst_piece_end = max(worst_piece_end, int((k_off[live] + 8).max()), int((v_off[live] + 8).max()))
             lds = ((tid // 64) + j * TW) * 512 + (tid % 64) * 8 + 8      # elements: base of the wave's fetch + lane * 16 B
@@ -97,6 +98,38 @@ def tile_extents(HD, kvh_count, tiles, positions, lp, table_width):
     assert worst_page_index < table_width
     assert worst_piece_end <= page_stride
     return worst_page_index, worst_piece_end, worst_lds_end, TCH * 8
+
+
+# The statements of the kernel source that the functions here repeat. If one of them is edited there, the test below
+# fails until the model has been brought in step with it (and this list with the source).
+MIRRORED = {
+    "attention_mfma.hip": [
+        "const int key_in_tile = (c & 3) | ((c & 4) << 1) | ((c & 8) >> 1);",
+        "k_off[j] = (unsigned)k_head + key_in_tile * HD + ((c >> 4) % NCH) * 8;",
+        "v_off[j] = (unsigned)v_head + (((c >> 5) % DB) * 16 + (c & 15)) * page_size + ((c >> 4) & 1) * 8;",
+        "const int key0 = k_lo + (2 * s0 + lane) * 16;",
+        "const int pg = bt[key0 < k_hi ? (PS16 ? key0 >> 4 : key0 / page_size) : 0];",
+        "const TileAddress* at = &run_tiles[wave][2 * (s - run_first)];",
+        "if (s - run_first >= 32) load_run(s);",
+        "const int item_splits = max(1, min(n_splits, (n_steps + max_steps - 1) / max_steps));",
+        "static constexpr int TPT = (TCH + TW * 64 - 1) / (TW * 64);",
+        "&k_lds[buf][(wave + j * TW) * 512]",
+        # the one-wave kernel
+        "const bf16* kp = base + k_head + (long)(slot0 + c16) * HD;",
+        "const bf16* vp = base + v_head + (long)c16 * page_size + slot0 + g * 4;",
+        "const long page_stride = 2L * n_kv_heads * page_size * HD;",
+        "const long v_head = ((long)n_kv_heads + kvh) * page_size * HD;",
+    ],
+}
+
+
+def test_the_model_mirrors_the_kernel_source_as_it_is():
+    csrc = os.path.join(os.path.dirname(PRESETS), os.pardir, "csrc")
+    for name, statements in MIRRORED.items():
+        with open(os.path.join(csrc, name)) as f:
+            text = " ".join(f.read().split())
+        for st in statements:
+            assert " ".join(st.split()) in text, f"{name} no longer holds `{st}`: bring tests/test_address_model.py in step"
 
 
 def wave_extents(HD, kvh_count, items, positions, lp, single, table_width):

@@ -209,6 +209,51 @@ def test_single_rows_of_uneven_lengths_behind_a_window(ops_for, window):
         torch.testing.assert_close(got[i].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,window,tile_splits", [(12, 3, 128, 0, False), (12, 3, 128, 0, True), (8, 2, 64, 700, False)])
+def test_decoded_rows_of_uneven_lengths_beside_a_portions_tiles(ops_for, monkeypatch, n_heads, n_kv, hd, window, tile_splits):
+    """A step as serving brings them: a prompt's portion, which goes to tiles, in the middle of decoded tokens of
+    requests that differ widely in length, whose key splits are then planned row by row although the step is not one
+    of single rows alone. The planned entries name the rows' lines of the block table, which are no longer 0, 1, ...;
+    partial results of both kernels share the workspace and the merge."""
+    from tiny_inference_server_amd.ops import hip_ops
+    if tile_splits:
+        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_FROM", 4)
+        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_SHARE", 1.0)
+    ops = ops_for(torch.bfloat16)
+    page_size = 16
+    lens = [1, 5000, 17, 900, 33, 4096, 64, 2, 640]
+    lens_after = [31, 32, 2500, 7, 129, 1300, 151, 999, 3000, 45]
+    p0, n = 1000, 600                                            # the portion: request 9 of 19
+    kv_lens = lens + [p0 + n] + lens_after
+    seq_rows, first = [], 0
+    for i, L in enumerate(kv_lens):
+        rows = n if i == len(lens) else 1
+        seq_rows.append((first, L - rows, rows))
+        first += rows
+    R = first
+    group, cols = n_heads // n_kv, hip_ops.tile_columns(hd)
+    nb, items, tiles, steps = hip_ops.attention_items(seq_rows, group, cols, n_kv)
+    beside = hip_ops.planned_beside_tiles(seq_rows, items, tiles, n_heads, n_kv, hd, window)
+    assert beside is not None and len(tiles) == -(-n // (4 * (cols // group)))
+    live = beside[0][beside[0][:, 0] >= 0]
+    assert sorted(set(live[:, 3].tolist())) == [i for i in range(len(kv_lens)) if i != len(lens)]
+    assert (live[:, 1] >> 16).max() > 1                           # some row is cut, so partial results are merged
+    plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page_size, torch.bfloat16, seed=29)
+    positions, row_seq = [], []
+    for i, (f, q0, rows) in enumerate(seq_rows):
+        positions += list(range(q0, q0 + rows)); row_seq += [i] * rows
+    q = rnd((R, n_heads * hd), torch.bfloat16, 30)
+    batch = SimpleNamespace(positions=torch.tensor(positions, dtype=torch.int32).cuda(),
+                            row_seq=torch.tensor(row_seq, dtype=torch.int32).cuda(),
+                            block_tables={"g": tables.cuda()}, max_kv_len=max(kv_lens), extras={},
+                            n_rows=R, max_seq_rows=n, seq_rows=seq_rows)
+    got = ops.paged_attention(q.cuda(), plane.cuda(), batch, "g", n_heads, n_kv, hd, window=window).cpu()
+    assert torch.isfinite(got.float()).all()
+    for r in list(range(len(lens))) + list(range(len(lens), len(lens) + n, 7)) + list(range(len(lens) + n - 2, R)):
+        want = dense_reference(q[r].view(n_heads, hd), ks[row_seq[r]], vs[row_seq[r]], group, positions[r], window)
+        torch.testing.assert_close(got[r].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("page_size", [16, 32])
 def test_single_rows_walking_a_long_context_without_splits(ops_for, monkeypatch, page_size):
     """With no key splits one wave walks a request's whole context alone: thousands of keys, hundreds of steps,

@@ -938,15 +938,15 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
     return tis_fail("attention_mfma: bad grid %d x %d (tiles: %d)", n_kv_heads, n_splits, tile_splits);
   const int stride = split_stride(n_items, n_tiles, n_splits, tile_splits);
   if (stride > 1 && (!part_o || !part_ml)) return tis_fail("attention_mfma: %d splits need a workspace", stride);
-  if (min_steps < -1 || (min_steps == -1 && (!items || n_items < 1 || n_tiles > 0)))
-    return tis_fail("attention_mfma: min_steps=%d; -1 goes with a planned list of single rows and no tiles", min_steps);
+  if (min_steps < -1 || (min_steps == -1 && (!items || n_items < 1)))
+    return tis_fail("attention_mfma: min_steps=%d; -1 goes with a planned list of single rows", min_steps);
   if (min_steps == -1 && ((uintptr_t)items % 16))
     return tis_fail("attention_mfma: a planned list's entries of four integers must be 16-byte aligned");
   if (min_steps != 0 && n_splits > 1 && !row_splits)
     return tis_fail("attention_mfma: splits chosen item by item (min_steps=%d) need the per-row count array", min_steps);
   if (n_tiles > 0 && tile_max_steps < 1) return tis_fail("attention_mfma: a tile's splits need a longest chain of at least one step");
-  if (n_tiles > 0 && stride > 1 && (!row_splits || (n_items > 0 && min_steps < 1)))
-    return tis_fail("attention_mfma: tiles beside split key ranges need the per-row count array and a minimum of steps");
+  if (n_tiles > 0 && stride > 1 && (!row_splits || (n_items > 0 && min_steps == 0)))
+    return tis_fail("attention_mfma: tiles beside split key ranges need the per-row count array, and items that take their splits by their own length");
   if (stride == 1 || (n_tiles == 0 && min_steps == 0)) row_splits = nullptr;
   if ((q_ld % 8) || (out_ld % 4) || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)plane % 16))
     return tis_fail("attention_mfma: q, out and the cache plane must be 16-byte aligned with row strides in steps of 8");
@@ -967,6 +967,9 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
   }
   // From here on the second stream hangs off the first: whatever happens, it is joined again before this function
   // returns, so that a stream capture never ends with a branch left open.
+  // (the items first: their single waves spread over the chip and leave every compute unit room for a tile's
+  // workgroup; tiles launched first fill the units' LDS and registers and the items wait for them to finish: 64 decoded
+  // tokens beside a 2,048-token prompt 180 instead of 122 us)
   if (n_items > 0) {
     dim3 grid(n_items, n_kv_heads, min_steps < 0 ? 1 : n_splits);
 #define LAUNCH(NBV, PSV)                                                                                              \

@@ -159,6 +159,7 @@ _ATTN_PLANNED_MAX_WAVES = 384   # ... and requests x key/value heads are at most
                                 # same splits for all, us: 3 kv heads, 96 requests 72 / 87, 64: 43 / 47, 24: 20.5 /
                                 # 24.6; 4 heads, 96: 100 / 103, 48: 39 / 43; 8 heads, 64: 126 / 124, 32: 53.5 / 60.6;
                                 # 1 head, 64: 19.8 / 21.0; with 8 requests 13.2 / 12.4 (3 heads), 23.6 / 21.8 (8)
+_ATTN_PLANNED_SHARE_BESIDE_TILES = 0.5   # ... of that target where the list runs beside a portion's tiles
 _ATTN_MIN_SPLIT_KEYS = 128      # a split shorter than this costs more in merging than it gains in spreading
 _ATTN_TILE_WAVES = 4            # waves of the workgroup that takes a tile of a long portion
 _ATTN_TILE_GROUPS = 512         # workgroups of the tile kernel that the chip runs side by side
@@ -285,11 +286,13 @@ def decode_items_most_splits(n_rows: int, n_heads: int, head_dim: int, workspace
 
 
 def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspace_floats=None, window: int = 0,
-                 units: int = _CHIP_UNITS):
+                 units: int = _CHIP_UNITS, table_lines=None, all_rows: int = 0, share: float = 1.0):
     """The work list of a step of single rows whose requests differ widely in length: one entry per wave (and
     key/value head), (row, split + 65536 * splits of the row, position, block-table line), so that every wave walks
     about the same number of keys; longest first; padded with row -1 to a length that depends on the number of rows
-    alone (a captured launch keeps its grid while the lengths change). Returns (int32 [capacity, 4], most splits)."""
+    alone (a captured launch keeps its grid while the lengths change). Returns (int32 [capacity, 4], most splits).
+    table_lines: the rows' lines of the block table where they are not simply 0, 1, ... (single rows beside portions
+    of other requests); all_rows: the rows of the whole step then (they share the workspace for partial results)."""
     n = len(seq_rows)
     rows = np.fromiter((f for f, _, _ in seq_rows), dtype=np.int64, count=n)
     pos = np.fromiter((p0 for _, p0, _ in seq_rows), dtype=np.int64, count=n)
@@ -298,8 +301,8 @@ def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspa
     first = np.maximum(0, pos - window + 1) & ~31 if window > 0 else 0
     steps = (pos + 32 - first) // 32
     fewest = max(1, _ATTN_MIN_SPLIT_KEYS // 32)
-    even = max(fewest, -(-int(steps.sum()) * n_kv_heads // planned_target_waves(n_kv_heads, units)))
-    most = decode_items_most_splits(n, n_heads, head_dim, workspace_floats)
+    even = max(fewest, -(-int(steps.sum()) * n_kv_heads // max(1, int(planned_target_waves(n_kv_heads, units) * share))))
+    most = decode_items_most_splits(max(n, all_rows), n_heads, head_dim, workspace_floats)
     splits = np.clip((steps + even // 2) // even, 1, np.minimum(steps, most))
     cap = decode_items_capacity(n, n_kv_heads, units)
     total = int(splits.sum())
@@ -316,8 +319,25 @@ def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspa
     out[:total, 0] = rows[who]
     out[:total, 1] = which + (splits[who] << 16)
     out[:total, 2] = pos[who]
-    out[:total, 3] = who
+    out[:total, 3] = who if table_lines is None else np.asarray(table_lines, dtype=np.int64)[who]
     return out, most
+
+
+def planned_beside_tiles(seq_rows, items, tiles, n_heads: int, n_kv_heads: int, head_dim: int, window: int = 0,
+                         units: int = _CHIP_UNITS):
+    """For a step whose portions all go to tiles and whose other rows are single rows of requests that differ widely
+    in length (decoded tokens beside a prompt's portion): the planned list of decode_items for those rows, or None.
+    With the same number of splits for every row the longest request's waves would run on alone, here beside the
+    tiles' workgroups; 64 decoded tokens at 512 to 8,000 keys beside a 2,048-token portion take 86 us planned alone
+    and well over 110 with equal splits (12 heads over 3)."""
+    if not len(tiles) or not len(items) or int(items[:, 1].max()) != 1 or n_heads // n_kv_heads > 64:
+        return None
+    singles = [(f, p0, 1) for f, p0, n in seq_rows if n == 1]
+    if len(singles) != len(items) or not uneven_lengths(singles, window) or not planned_list_pays(len(singles), n_kv_heads):
+        return None
+    lines = [i for i, (_, _, n) in enumerate(seq_rows) if n == 1]
+    return decode_items(singles, n_heads, n_kv_heads, head_dim, window=window, units=units, table_lines=lines,
+                        all_rows=sum(n for _, _, n in seq_rows), share=_ATTN_PLANNED_SHARE_BESIDE_TILES)
 
 
 class AttentionLaunch(NamedTuple):
@@ -459,11 +479,17 @@ class HipOps:
                 entries, most = decode_items(seq_rows, n_heads, n_kv_heads, head_dim, window=window, units=self.units)
                 return {("attention_decode_items", group, cols, n_kv_heads, window): (add(entries), len(entries), most)}
             nb, items, tiles, steps = attention_items(seq_rows, group, cols, n_kv_heads)
-            if nb <= 4 and (len(items) or len(tiles)):
+            beside = planned_beside_tiles(seq_rows, items, tiles, n_heads, n_kv_heads, head_dim, window, self.units)
+            if beside is not None:
+                # one array: the planned entries of four integers, then the tiles' lines of two
+                entries, most = beside
+                plans[("attention_items", group, cols, n_kv_heads, window)] = (
+                    add(np.concatenate((entries.reshape(-1), tiles.reshape(-1)))), len(entries), 1, len(tiles), steps, most)
+            elif nb <= 4 and (len(items) or len(tiles)):
                 # one array: the items' lines, then the tiles'
                 # (a mixer with a window plans for itself: its lists are the same, its keys are its own)
                 plans[("attention_items", group, cols, n_kv_heads, window)] = (add(np.concatenate((items, tiles))), len(items),
-                                                                       nb, len(tiles), steps)
+                                                                       nb, len(tiles), steps, 0)
         return plans
 
     # ---- helpers -------------------------------------------------------------------------------------
@@ -836,8 +862,16 @@ class HipOps:
                     planned = (torch.from_numpy(entries).reshape(-1).to(self.device), len(entries), most)
                 else:
                     nb, host_items, host_tiles, steps = attention_items(batch.seq_rows, group, cols)
-                    both = np.ascontiguousarray(np.concatenate((host_items, host_tiles)))
-                    plan = (torch.from_numpy(both).reshape(-1).to(self.device), len(host_items), nb, len(host_tiles), steps)
+                    beside = planned_beside_tiles(batch.seq_rows, host_items, host_tiles, n_heads, n_kv_heads, head_dim,
+                                                  int(window), self.units)
+                    if beside is not None:
+                        both = np.concatenate((beside[0].reshape(-1), host_tiles.reshape(-1)))
+                        plan = (torch.from_numpy(np.ascontiguousarray(both)).to(self.device), len(beside[0]), 1,
+                                len(host_tiles), steps, beside[1])
+                    else:
+                        both = np.ascontiguousarray(np.concatenate((host_items, host_tiles)))
+                        plan = (torch.from_numpy(both).reshape(-1).to(self.device), len(host_items), nb, len(host_tiles),
+                                steps, 0)
             planned_splits = 0
             if planned is not None:
                 # single rows with splits planned row by row: one entry of four integers per wave
@@ -850,11 +884,18 @@ class HipOps:
                 while group > 16 * nb:
                     nb *= 2
             else:
-                lines, n_items, nb, n_tiles, tile_steps = plan
+                lines, n_items, nb, n_tiles, tile_steps, planned_splits = plan
                 lines = lines.reshape(-1)
-                items = lines[:2 * n_items] if n_items else None
-                tiles = lines[2 * n_items:] if n_tiles else None
-                if batch.max_seq_rows <= 1 and n_items == n:
+                width = 4 if planned_splits else 2      # a planned entry, or an item's (first row, rows)
+                if lines.numel() < width * n_items + 2 * n_tiles:
+                    raise KernelError(f"attention: the work list holds {lines.numel()} integers for {n_items} items "
+                                      f"and {n_tiles} tiles")
+                items = lines[:width * n_items] if n_items else None
+                tiles = lines[width * n_items:] if n_tiles else None
+                if planned_splits:
+                    while group > 16 * nb:
+                        nb *= 2
+                elif batch.max_seq_rows <= 1 and n_items == n:
                     items = None        # single rows in order: the kernel needs no list
             lib = self._attn_mfma.get(head_dim)
             if lib is None:
@@ -878,10 +919,8 @@ class HipOps:
                 part_ml = self._workspace[lp.ml_offset:]
                 if lp.min_steps != 0 or n_tiles:
                     row_splits = self._workspace[lp.row_splits_offset:]
-            if (not planned_splits and lines.numel() < 2 * (n_items + n_tiles)) or lines.dtype != torch.int32 \
-                    or not lines.is_contiguous():
-                raise KernelError(f"attention: the work list holds {lines.numel()} entries for {n_items} items and "
-                                  f"{n_tiles} tiles")
+            if lines.dtype != torch.int32 or not lines.is_contiguous():
+                raise KernelError("attention: the work list must be contiguous 32-bit integers")
             lib.tis_attention_mfma(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0),
                                    _ptr(batch.row_seq), _ptr(batch.positions), _ptr(items), n_items, nb, _ptr(tiles),
                                    n_tiles, _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), n, n_heads,

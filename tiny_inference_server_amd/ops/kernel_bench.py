@@ -79,10 +79,17 @@ def attention_case(ops, a):
         batch.extras[("attention_decode_items", nh // kvh, tile_columns(hd), kvh, 0)] = (
             torch.from_numpy(entries).reshape(-1).to(ops.device), len(entries), most)
     else:
+        from .hip_ops import planned_beside_tiles
         nb, items, tiles, steps = attention_items(seq_rows, nh // kvh, 0 if a.no_tiles else tile_columns(hd),
                                                   0 if a.tiles else kvh)
-        both = torch.from_numpy(np.ascontiguousarray(np.concatenate((items, tiles)))).reshape(-1).to(ops.device)
-        batch.extras[("attention_items", nh // kvh, tile_columns(hd), kvh, 0)] = (both, len(items), nb, len(tiles), steps)
+        beside = None if a.same_splits else planned_beside_tiles(seq_rows, items, tiles, nh, kvh, hd, 0, ops.units)
+        if beside is not None:      # decoded tokens of uneven lengths beside a portion's tiles: as the engine plans them
+            both = np.concatenate((beside[0].reshape(-1), tiles.reshape(-1)))
+            plan = (torch.from_numpy(np.ascontiguousarray(both)).to(ops.device), len(beside[0]), 1, len(tiles), steps, beside[1])
+        else:
+            both = torch.from_numpy(np.ascontiguousarray(np.concatenate((items, tiles)))).reshape(-1).to(ops.device)
+            plan = (both, len(items), nb, len(tiles), steps, 0)
+        batch.extras[("attention_items", nh // kvh, tile_columns(hd), kvh, 0)] = plan
     us = graph_time(lambda: ops.paged_attention(q, plane, batch, "g", nh, kvh, hd), a.reps)
     kv_bytes = sum(p0 + n for p0, n in segs) * kvh * hd * 2 * 2
     flops = sum(4 * nh * hd * (n * p0 + n * (n + 1) / 2) for p0, n in segs)

@@ -216,9 +216,9 @@ def test_decoded_rows_of_uneven_lengths_beside_a_portions_tiles(ops_for, monkeyp
     of single rows alone. The planned entries name the rows' lines of the block table, which are no longer 0, 1, ...;
     partial results of both kernels share the workspace and the merge."""
     from tiny_inference_server_amd.ops import hip_ops
+    monkeypatch.setattr(hip_ops, "_ATTN_PLANNED_BESIDE_FROM", 0.0)    # (whether or not the estimate says it pays here)
     if tile_splits:
-        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_FROM", 4)
-        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_SHARE", 1.0)
+        monkeypatch.setattr(hip_ops, "_tiles_cut_pays", lambda *a: True)
     ops = ops_for(torch.bfloat16)
     page_size = 16
     lens = [1, 5000, 17, 900, 33, 4096, 64, 2, 640]
@@ -233,7 +233,7 @@ def test_decoded_rows_of_uneven_lengths_beside_a_portions_tiles(ops_for, monkeyp
     R = first
     group, cols = n_heads // n_kv, hip_ops.tile_columns(hd)
     nb, items, tiles, steps = hip_ops.attention_items(seq_rows, group, cols, n_kv)
-    beside = hip_ops.planned_beside_tiles(seq_rows, items, tiles, n_heads, n_kv, hd, window)
+    beside = hip_ops.planned_beside_tiles(seq_rows, items, tiles, steps, n_heads, n_kv, hd, window)
     assert beside is not None and len(tiles) == -(-n // (4 * (cols // group)))
     live = beside[0][beside[0][:, 0] >= 0]
     assert sorted(set(live[:, 3].tolist())) == [i for i in range(len(kv_lens)) if i != len(lens)]
@@ -345,8 +345,7 @@ def test_long_portions_by_tiles(ops_for, monkeypatch, n_heads, n_kv, hd, page_si
     from tiny_inference_server_amd.ops import hip_ops
     from tiny_inference_server_amd.ops.hip_ops import attention_items, tile_columns
     if splits:
-        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_FROM", 4)
-        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_SHARE", 1.0)
+        monkeypatch.setattr(hip_ops, "_tiles_cut_pays", lambda *a: True)
     ops = ops_for(torch.bfloat16)
     group = n_heads // n_kv
     tile_rows = 4 * (tile_columns(hd) // group)
@@ -382,8 +381,7 @@ def test_a_tile_sees_a_far_key_and_a_rows_own_key(ops_for, monkeypatch, splits):
     through."""
     from tiny_inference_server_amd.ops import hip_ops
     if splits:
-        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_FROM", 4)
-        monkeypatch.setattr(hip_ops, "_ATTN_TILE_SPLIT_SHARE", 1.0)
+        monkeypatch.setattr(hip_ops, "_tiles_cut_pays", lambda *a: True)
     ops = ops_for(torch.bfloat16)
     n_heads, n_kv, hd, page_size, L = 4, 1, 64, 16, 1200
     plane, tables, ks, vs = make_paged([L], n_kv, hd, page_size, torch.bfloat16, seed=38)

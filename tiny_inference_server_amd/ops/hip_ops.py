@@ -159,19 +159,25 @@ _ATTN_PLANNED_MAX_WAVES = 384   # ... and requests x key/value heads are at most
                                 # same splits for all, us: 3 kv heads, 96 requests 72 / 87, 64: 43 / 47, 24: 20.5 /
                                 # 24.6; 4 heads, 96: 100 / 103, 48: 39 / 43; 8 heads, 64: 126 / 124, 32: 53.5 / 60.6;
                                 # 1 head, 64: 19.8 / 21.0; with 8 requests 13.2 / 12.4 (3 heads), 23.6 / 21.8 (8)
-_ATTN_PLANNED_SHARE_BESIDE_TILES = 0.5   # ... of that target where the list runs beside a portion's tiles
+_ATTN_DECODE_BYTES_PER_US = 5.0e6   # keys and values a step of decoded tokens streams: 5 TB/s
+_ATTN_PLANNED_BESIDE_FROM = 1.15   # single rows beside tiles get a planned list if they take this much longer than the tiles
+_ATTN_PLANNED_WAVES_BESIDE_TILES = 1.5   # ... and at this many waves per compute unit, over all key/value heads, where
+                                # the list runs beside a portion's tiles, whose workgroups need room on every unit
 _ATTN_MIN_SPLIT_KEYS = 128      # a split shorter than this costs more in merging than it gains in spreading
 _ATTN_TILE_WAVES = 4            # waves of the workgroup that takes a tile of a long portion
 _ATTN_TILE_GROUPS = 512         # workgroups of the tile kernel that the chip runs side by side
 _ATTN_TILE_MIN_STEPS = 8        # steps of 32 keys below which a tile's split is not worth its merge
 _ATTN_TILE_SPLIT_SLACK = 1.4    # a split may be this much longer than an even share of all steps
-_ATTN_TILE_SPLIT_FROM = 40      # tiles are cut into key splits only if the longest walks at least this many steps ...
-_ATTN_TILE_SPLIT_SHARE = 0.3    # ... and an even share of all steps is at most this fraction of it: a few long chains.
-                                # Otherwise the merge (a launch, and 32-bit partial results written and read) costs
-                                # more than shorter chains save. 12 heads of 128 over 3, us, splits / none / one-wave
-                                # kernel: 4 prompts of 512 tokens 28.8 / 18.8 / 22.8, 8 of 512 40.8 / 25.4 / 33.2, 4 of
-                                # 1,024 50.6 / 39.5 / 57.2, one of 1,024 29.2 / 28.6 / 29.2; but one of 1,536 35.3 /
-                                # 39.9 / 47.7, of 2,048 42.4 / 51.3 / 69.5, 512 tokens behind 3,000 41.5 / 82.5 / 60.0
+_ATTN_TILE_STEP_US = (0.72, 1.3)   # what a tile's step of 32 keys takes while a workgroup has a compute unit to itself,
+                                # and once two share one (12 heads of 128 over 3; other geometries differ little)
+_ATTN_TILE_MERGE_US = (10.0, 4.0, 6e6)   # what cutting tiles into key splits costs beyond the tiles' own time: the
+                                # merge's launch and the per-row counts (less where the items' splits are merged anyway),
+                                # and microseconds per byte of 32-bit partial results. Tiles are cut only where, by
+                                # these figures, the shorter chains save more than that. 12 heads of 128 over 3, us,
+                                # cut / uncut / one-wave kernel: 4 prompts of 512 tokens 28.8 / 18.8 / 22.8, 8 of 512
+                                # 40.8 / 25.4 / 33.2, 4 of 1,024 50.6 / 39.5 / 57.2, one of 1,024 29.2 / 28.6 / 29.2; but
+                                # one of 1,536 35.3 / 39.9 / 47.7, of 2,048 42.4 / 51.3 / 69.5, 512 tokens behind 3,000
+                                # others 41.5 / 82.5 / 60.0
 _ATTN_TILE_PARTIAL_BYTES = 40 << 20   # partial results (32-bit, per split) beyond which the merge costs more than
                                       # shorter chains save; at least two splits are always allowed
 _ATTN_TILE_MIN_WORK_MIXED = 1500   # tile steps times key/value heads below which the one-wave kernel is the faster
@@ -323,21 +329,39 @@ def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspa
     return out, most
 
 
-def planned_beside_tiles(seq_rows, items, tiles, n_heads: int, n_kv_heads: int, head_dim: int, window: int = 0,
-                         units: int = _CHIP_UNITS):
+def planned_beside_tiles(seq_rows, items, tiles, tile_steps, n_heads: int, n_kv_heads: int, head_dim: int,
+                         window: int = 0, units: int = _CHIP_UNITS):
     """For a step whose portions all go to tiles and whose other rows are single rows of requests that differ widely
     in length (decoded tokens beside a prompt's portion): the planned list of decode_items for those rows, or None.
     With the same number of splits for every row the longest request's waves would run on alone, here beside the
-    tiles' workgroups; 64 decoded tokens at 512 to 8,000 keys beside a 2,048-token portion take 86 us planned alone
-    and well over 110 with equal splits (12 heads over 3)."""
-    if not len(tiles) or not len(items) or int(items[:, 1].max()) != 1 or n_heads // n_kv_heads > 64:
+    tiles' workgroups. It pays where the single rows are the longer half of the pair: beside tiles that take as long as
+    they do or longer (a portion deep in a long prompt) the rows are done first either way, and the list only costs the
+    host its making. 64 decoded tokens at 512 to 8,000 keys, us a layer, planned / same splits for all, 12 heads over 3:
+    beside a 2,048-token prompt 125 / 151, beside 1,024 tokens behind 1,000 others 126 / 151, beside 2,048 behind
+    2,048 others 143 / 154; 16 over 4: 158 / 191, 164 / 195 and 197 / 186."""
+    n_items = len(items)
+    if not len(tiles) or n_items < _ATTN_PLANNED_MIN_ROWS or n_items * n_kv_heads > _ATTN_PLANNED_MAX_WAVES \
+            or n_heads // n_kv_heads > 64 or int(items[:, 1].max()) != 1:
         return None
-    singles = [(f, p0, 1) for f, p0, n in seq_rows if n == 1]
-    if len(singles) != len(items) or not uneven_lengths(singles, window) or not planned_list_pays(len(singles), n_kv_heads):
+    singles, lines, all_rows = [], [], 0
+    for i, (f, p0, n) in enumerate(seq_rows):
+        all_rows += n
+        if n == 1:
+            singles.append((f, p0, 1))
+            lines.append(i)
+    if len(singles) != n_items or not uneven_lengths(singles, window):
         return None
-    lines = [i for i, (_, _, n) in enumerate(seq_rows) if n == 1]
+    # what the rows take at the rate a step of decoded tokens streams keys and values, against the tiles' estimate
+    row_steps = sum((p0 + 32) >> 5 if window <= 0 or p0 < window else (p0 + 32 - ((p0 - window + 1) & ~31)) >> 5
+                    for _, p0, _ in singles)
+    rows_us = row_steps * n_kv_heads * 64 * head_dim * 2 / _ATTN_DECODE_BYTES_PER_US
+    cut, cut_steps = _tiles_cut(all_rows, len(tiles), tile_steps, n_heads, n_kv_heads, head_dim)
+    tiles_us = min(_tiles_us(all_rows, len(tiles), tile_steps[0], tile_steps[1], cut, cut_steps, n_heads, n_kv_heads,
+                             head_dim, True, units))
+    if rows_us < _ATTN_PLANNED_BESIDE_FROM * tiles_us:
+        return None
     return decode_items(singles, n_heads, n_kv_heads, head_dim, window=window, units=units, table_lines=lines,
-                        all_rows=sum(n for _, _, n in seq_rows), share=_ATTN_PLANNED_SHARE_BESIDE_TILES)
+                        all_rows=all_rows, share=min(1.0, _ATTN_PLANNED_WAVES_BESIDE_TILES / n_kv_heads))
 
 
 class AttentionLaunch(NamedTuple):
@@ -352,6 +376,37 @@ class AttentionLaunch(NamedTuple):
     ml_offset: int
     row_splits_offset: int
     need_floats: int
+
+
+def _tiles_us(n, n_tiles, all_steps, longest, cut, cut_steps, n_heads, n_kv_heads, head_dim, merged_anyway, units):
+    """Estimated microseconds of a call's tiles left whole, and cut into `cut` key splits of at most `cut_steps` steps:
+    the longest chain of steps sets the time (a step takes longer once two workgroups share a compute unit, and no
+    less than all steps spread evenly take), and the cut adds the merge."""
+    alone, shared = _ATTN_TILE_STEP_US
+
+    def chain_us(steps, workgroups):
+        return max(steps * min(shared, alone * max(1.0, workgroups / units)), all_steps * n_kv_heads / (2 * units) * shared)
+    whole = chain_us(longest, n_tiles * n_kv_heads)
+    launch, launch_merged, bytes_per_us = _ATTN_TILE_MERGE_US
+    merge = (launch_merged if merged_anyway else launch) + n * n_heads * head_dim * 4 * cut / bytes_per_us
+    parts = chain_us(cut_steps, n_kv_heads * (all_steps / cut_steps + n_tiles / 2)) + merge
+    return whole, parts
+
+
+def _tiles_cut_pays(*args) -> bool:
+    """Whether cutting the tiles of a call into key splits is estimated to be faster than leaving them whole."""
+    whole, parts = _tiles_us(*args)
+    return parts < whole
+
+
+def _tiles_cut(n, n_tiles, tile_steps, n_heads, n_kv_heads, head_dim):
+    """Into how many key splits, of at most how many steps, a call's tiles would be cut if they are cut."""
+    all_steps, longest = tile_steps
+    share = all_steps * n_kv_heads / _ATTN_TILE_GROUPS
+    cut_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
+    most_splits = max(2, _ATTN_TILE_PARTIAL_BYTES // (n * n_heads * head_dim * 4))
+    cut = max(1, min(most_splits, -(-longest // cut_steps)))
+    return cut, max(cut_steps, -(-longest // cut))
 
 
 def attention_launch_plan(n, n_items, n_tiles, tile_steps, single, max_kv_len, n_heads, n_kv_heads, head_dim,
@@ -387,12 +442,10 @@ def attention_launch_plan(n, n_items, n_tiles, tile_steps, single, max_kv_len, n
         # of 128 (tiles / one-wave kernel, us): 2,048 rows from 0: 54 / 69; from 2,048: 99 / 134; from 6,144:
         # 196 / 260; 4,096 rows: 146 / 202.
         all_steps, longest = tile_steps
-        share = all_steps * n_kv_heads / _ATTN_TILE_GROUPS
-        if longest >= _ATTN_TILE_SPLIT_FROM and share <= _ATTN_TILE_SPLIT_SHARE * longest:
-            tile_max_steps = max(_ATTN_TILE_MIN_STEPS, int(share * _ATTN_TILE_SPLIT_SLACK) + 1)
-            most_splits = max(2, _ATTN_TILE_PARTIAL_BYTES // (n * n_heads * head_dim * 4))
-            tile_splits = max(1, min(most_splits, -(-longest // tile_max_steps)))
-            tile_max_steps = max(tile_max_steps, -(-longest // tile_splits))
+        cut, cut_steps = _tiles_cut(n, n_tiles, tile_steps, n_heads, n_kv_heads, head_dim)
+        if cut > 1 and _tiles_cut_pays(n, n_tiles, all_steps, longest, cut, cut_steps, n_heads, n_kv_heads, head_dim,
+                                       n_splits > 1, units):
+            tile_splits, tile_max_steps = cut, cut_steps
     # partial results of split key ranges live in one workspace of fixed size; fewer splits where it
     # would not suffice
     most = max(1, (workspace_floats - n) // (n * n_heads * (head_dim + 2)))
@@ -479,7 +532,7 @@ class HipOps:
                 entries, most = decode_items(seq_rows, n_heads, n_kv_heads, head_dim, window=window, units=self.units)
                 return {("attention_decode_items", group, cols, n_kv_heads, window): (add(entries), len(entries), most)}
             nb, items, tiles, steps = attention_items(seq_rows, group, cols, n_kv_heads)
-            beside = planned_beside_tiles(seq_rows, items, tiles, n_heads, n_kv_heads, head_dim, window, self.units)
+            beside = planned_beside_tiles(seq_rows, items, tiles, steps, n_heads, n_kv_heads, head_dim, window, self.units)
             if beside is not None:
                 # one array: the planned entries of four integers, then the tiles' lines of two
                 entries, most = beside
@@ -862,8 +915,8 @@ class HipOps:
                     planned = (torch.from_numpy(entries).reshape(-1).to(self.device), len(entries), most)
                 else:
                     nb, host_items, host_tiles, steps = attention_items(batch.seq_rows, group, cols)
-                    beside = planned_beside_tiles(batch.seq_rows, host_items, host_tiles, n_heads, n_kv_heads, head_dim,
-                                                  int(window), self.units)
+                    beside = planned_beside_tiles(batch.seq_rows, host_items, host_tiles, steps, n_heads, n_kv_heads,
+                                                  head_dim, int(window), self.units)
                     if beside is not None:
                         both = np.concatenate((beside[0].reshape(-1), host_tiles.reshape(-1)))
                         plan = (torch.from_numpy(np.ascontiguousarray(both)).to(self.device), len(beside[0]), 1,

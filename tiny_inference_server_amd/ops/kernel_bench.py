@@ -82,7 +82,7 @@ def attention_case(ops, a):
         from .hip_ops import planned_beside_tiles
         nb, items, tiles, steps = attention_items(seq_rows, nh // kvh, 0 if a.no_tiles else tile_columns(hd),
                                                   0 if a.tiles else kvh)
-        beside = None if a.same_splits else planned_beside_tiles(seq_rows, items, tiles, nh, kvh, hd, 0, ops.units)
+        beside = None if a.same_splits else planned_beside_tiles(seq_rows, items, tiles, steps, nh, kvh, hd, 0, ops.units)
         if beside is not None:      # decoded tokens of uneven lengths beside a portion's tiles: as the engine plans them
             both = np.concatenate((beside[0].reshape(-1), tiles.reshape(-1)))
             plan = (torch.from_numpy(np.ascontiguousarray(both)).to(ops.device), len(beside[0]), 1, len(tiles), steps, beside[1])

@@ -641,6 +641,35 @@ def test_product_with_norm_residual_and_gate_for_many_rows(ops_for, M, N, K):
             assert torch.equal(again[r + shift], normed[r])
 
 
+@pytest.mark.parametrize("M", [129, 200, 777, 2049])
+@pytest.mark.parametrize("N,K", [(64, 8), (132, 72), (520, 1528), (1536, 640), (4096, 4096), (6148, 200)])
+def test_tiled_product_at_widths_the_library_is_not_used_at(ops_for, M, N, K):
+    """Many rows at a width outside the library's list go to the tiled product of this repository: row and column
+    counts that end inside a tile, a K that ends inside a step of 64 (down to a single piece of 8), tiles of 64 and of
+    128 columns, with a residual that is the output itself or another tensor. Against exact sums of the same bfloat16
+    operands; and a row's result does not depend on which tile or rows it shares."""
+    from tiny_inference_server_amd.ops.hip_ops import product_route
+    ops = ops_for(torch.bfloat16)
+    assert product_route(M, N, K, True, False, ops.library_widths, ops.few_rows) == "tiles"
+    x, w = rnd((M, K), torch.bfloat16, 60, 1.0), rnd((N, K), torch.bfloat16, 61, K ** -0.5)
+    res = rnd((M, N), torch.bfloat16, 62)
+    want = x.double() @ w.double().t()
+    t = dict(rtol=8e-3, atol=4e-3)
+    got = ops.linear(x.cuda(), w.cuda())
+    torch.testing.assert_close(got.cpu().double(), want, **t)
+    torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), residual=res.cuda()).cpu().double(), want + res.double(), **t)
+    # the residual as the output's own memory
+    out, xd, wd = res.clone().cuda(), x.cuda(), w.cuda()
+    ops.gemm_tiles.tis_gemm_tiles(xd.data_ptr(), K, wd.data_ptr(), out.data_ptr(), N, out.data_ptr(), N, M, N, K,
+                                  ops._stream())
+    torch.testing.assert_close(out.cpu().double(), want + res.double(), **t)
+    # a row moved to another place among other rows gives the same bits
+    others = rnd((M, K), torch.bfloat16, 63, 2.0)
+    others[M - 1] = x[3]
+    again = ops.linear(others.cuda(), w.cuda())
+    assert torch.equal(again[M - 1].cpu(), got[3].cpu())
+
+
 def test_library_product_at_listed_widths(ops_for):
     """Every width that may go to the library's product (ops/library_widths.json), at row counts as serving brings
     them: a few more than the few-row kernel takes, a portion beside decoded tokens, a prediction head's rows one

@@ -35,7 +35,7 @@ def host_ops(widths=None, few_rows=hip_ops._FEW_ROWS):
     ops.library_widths = library_widths() if widths is None else frozenset(widths)
     ops._warned_widths = set()
     ops.calls = []
-    for lib in ("rowwise", "gemm_skinny", "gemm_library", "gemm_plain"):
+    for lib in ("rowwise", "gemm_skinny", "gemm_library", "gemm_plain", "gemm_tiles"):
         setattr(ops, lib, Recorder(ops.calls, lib))
     ops._stream = lambda: c_void_p(0)
     return ops
@@ -65,7 +65,9 @@ def test_routes():
     assert product_route(hip_ops._FEW_ROWS, 2304, 1536, True, False, w) == "few_rows"
     assert product_route(hip_ops._FEW_ROWS + 1, 2304, 1536, True, False, w) == "library"
     assert product_route(2048, 2304, 1536, True, True, w) == "few_rows"         # 32-bit results: own kernels
-    assert product_route(2048, 6144, 4096, True, False, w) == "few_rows"        # a width nobody listed
+    assert product_route(2048, 6144, 4096, True, False, w) == "tiles"           # a width nobody listed: own kernel
+    assert product_route(128, 6144, 4096, True, False, w) == "few_rows"
+    assert product_route(2048, 6146, 4096, True, False, w) == "few_rows"        # ... whose stores need N in steps of 4
     assert product_route(2048, 2304, 1536, False, False, w) == "plain"
 
 
@@ -114,9 +116,14 @@ def test_no_unlisted_width_and_no_unrounded_row_count_reaches_the_library(seed):
             # the operands reach as far as the rows asked for, in memory that is theirs
             assert X % 16 == 0 and W % 16 == 0 and C % 16 == 0 and R % 16 == 0
             assert x_ld >= K and c_ld >= N
+        elif fn == "tis_gemm_tiles":
+            X, x_ld, W, R, r_ld, C, c_ld, rows, n, k = a[:10]
+            assert (rows, n, k) == (M, N, K) and (N, K) not in library_widths() and M > ops.few_rows
+            assert K % 8 == 0 and N % 4 == 0 and X % 16 == 0 and W % 16 == 0 and C % 8 == 0 and R % 8 == 0
+            assert C == out.data_ptr() and inside(out, C, M, c_ld, N) and x_ld >= K
         else:
             assert fn == "tis_gemm_skinny", fn
-            assert M <= ops.few_rows or (N, K) not in library_widths()
+            assert M <= ops.few_rows or ((N, K) not in library_widths() and N % 4)
 
 
 def test_rows_beyond_a_callers_tensor_are_never_read():
@@ -160,5 +167,8 @@ def test_gated_and_projection_products_follow_the_same_routes():
     assert [c for c in ops.calls if c[0] == "tis_gemm_library"][0][1][7] == 2304
     ops.calls.clear()
     ops.linear_swiglu(ops.empty(2112, 4096), torch.empty(28672, 4096, dtype=torch.bfloat16), rms=(torch.ones(4096), 1e-5))
-    assert [c[0] for c in ops.calls] == ["tis_gemm_skinny"]           # norm and gate fused, rows in panels
+    assert [c[0] for c in ops.calls] == ["tis_rmsnorm", "tis_gemm_tiles", "tis_swiglu"]    # an unlisted width: own tiles
+    ops.calls.clear()
+    ops.linear_swiglu(ops.empty(100, 4096), torch.empty(28672, 4096, dtype=torch.bfloat16), rms=(torch.ones(4096), 1e-5))
+    assert [c[0] for c in ops.calls] == ["tis_gemm_skinny"]           # few rows: norm and gate fused
     assert hip_ops._FEW_ROWS == ops.few_rows

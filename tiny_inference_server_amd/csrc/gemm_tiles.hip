@@ -1,0 +1,196 @@
+// C[M,N] = X[M,K] . W[N,K]^T (+ R[M,N]) in bfloat16 for many rows at widths where the library's product is not used:
+// a product tiled in both directions on v_mfma_f32_32x32x16_bf16 (gfx950), operands through LDS by direct loads.
+// (The few-row kernel takes such a product in panels of 32 rows, each of which streams all of W again: 0.25 to 0.3
+// PFLOP/s at 2,048 rows. This kernel reaches 0.45 to 0.95 on the same shapes; the library's kernels, where they may be
+// used, 0.5 to 1.3.) The reference's engine uses a library product here (x @ W, main_models_new.py:19-20).
+//
+// A workgroup of four waves (2 x 2) owns a tile of 128 rows x 128 or 64 columns and walks K in steps of 64. A step's
+// operand rows, 128 bytes each, are copied into LDS by global_load_lds_dwordx4 (no registers; eight lanes read one
+// row's 128 bytes), one step ahead of the products, into one of two buffers; two workgroups share a compute unit and
+// fill each other's waits. A row's eight 16-byte pieces lie in LDS with their index XORed by the row's number, so
+// that the 32 rows an operand fetch reads for one piece index fall into different banks; the copying lane picks the
+// piece that belongs in its slot. The result tile is computed transposed (W's rows are the first operand), so that a
+// lane ends up with four consecutive columns of one row: 8-byte stores, and the residual read the same way.
+// A row's sums run over K in the same order whatever M is: its result does not depend on the other rows.
+#include "common.h"
+
+TIS_DEFINE_LAST_ERROR(tis_gemm_tiles)
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+static constexpr int GT_BM = 128, GT_BK = 64, GT_WAVES = 4, GT_PIECES = GT_BK / 8;
+
+// what lanes past the end of K read in the last step: zeros
+static __device__ __attribute__((aligned(16))) unsigned char gt_zeros[16];
+
+#pragma clang diagnostic ignored "-Winline-asm"   // M0 in a clobber list: meant
+// One 16-byte piece per lane from global memory straight into LDS: lane i's piece lands at lds_addr + 16 * i. In
+// assembly, because the compiler would order every later LDS read behind such a load, whichever buffer it reads; so
+// the compiler does not count these loads either, and whoever reads the pieces waits for them (vmcnt) and for the
+// other waves (barrier).
+__device__ __forceinline__ void gt_copy16(const void* scalar_src, unsigned lane_bytes, unsigned lds_addr) {
+  const uint64_t a = (uint64_t)scalar_src;
+  const uint64_t sc = ((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(a >> 32)) << 32) |
+                      (unsigned)__builtin_amdgcn_readfirstlane((int)a);
+  const unsigned base = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_addr);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_bytes), "s"(sc), "s"(base) : "memory", "m0");
+}
+// the same with every lane's own address
+__device__ __forceinline__ void gt_copy16(const void* lane_src, unsigned lds_addr) {
+  const unsigned base = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_addr);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(lane_src), "s"(base) : "memory", "m0");
+}
+
+template <int BN, bool RESIDUAL>
+__global__ __launch_bounds__(GT_WAVES * 64) void gemm_tiles_kernel(
+    const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const bf16* R, long r_ld, bf16* C, long c_ld,
+    int M, int N, int K) {
+  constexpr int BM = GT_BM, BK = GT_BK, PCS = GT_PIECES, ROWS = BM + BN;
+  constexpr int STAGE = ROWS * BK * 2;                  // bytes of a buffer: X's rows, then W's
+  constexpr int LPW = ROWS * PCS / 64 / GT_WAVES;       // loads of a step that each wave issues, 8 rows each
+  constexpr int TM = BM / 2 / 32, TN = BN / 2 / 32;     // 32 x 32 result tiles of a wave
+  static_assert(ROWS * PCS % (64 * GT_WAVES) == 0 && TN >= 1, "tile sizes");
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * STAGE];
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, r32 = lane & 31, h = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_m = (M + BM - 1) / BM;
+  const long m0 = (long)(blockIdx.x % tiles_m) * BM, n0 = (long)(blockIdx.x / tiles_m) * BN;
+  const unsigned lds0 = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds;
+
+  // The wave's loads of a step: load j brings rows 8 (wave * LPW + j) .. +7 of the buffer, lane (row, slot) the piece
+  // slot ^ (row & 7) of its row. Rows past the matrix's last are the last row again (their results are not stored).
+  const unsigned char* first_row[LPW];       // of the load's first row, at K offset 0 (the same on all lanes)
+  unsigned lane_off[LPW];                    // the lane's piece from there, in bytes
+  int lane_piece;                            // which 8 elements of a step's 64 the lane brings
+  {
+    const int slot = lane & 7;
+    lane_piece = slot ^ ((lane >> 3) & 7);   // (a load's first row is a multiple of 8)
+  }
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) {
+    const int row0 = (wave * LPW + j) * 8, row = row0 + (lane >> 3);
+    const bool of_x = row0 < BM;
+    const long ld = of_x ? x_ld : (long)K;
+    const long last = of_x ? (long)M - 1 : (long)N - 1;
+    const long g_first = min(last, of_x ? m0 + row0 : n0 + (row0 - BM));
+    const long g_row = min(last, of_x ? m0 + row : n0 + (row - BM));
+    first_row[j] = (const unsigned char*)(of_x ? X : W) + g_first * ld * 2;
+    lane_off[j] = (unsigned)((g_row - g_first) * ld * 2 + lane_piece * 16);
+  }
+  auto stage = [&](int k0, int buf) {
+#pragma unroll
+    for (int j = 0; j < LPW; ++j)
+      gt_copy16(first_row[j] + (long)k0 * 2, lane_off[j], lds0 + buf * STAGE + (wave * LPW + j) * 1024);
+  };
+  // the last step of a K that is no multiple of 64: pieces past the end come from a block of zeros
+  auto stage_tail = [&](int k0, int buf) {
+    const bool inside = k0 + lane_piece * 8 < K;
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) {
+      const unsigned char* src = inside ? first_row[j] + (long)k0 * 2 + lane_off[j] : gt_zeros;
+      gt_copy16(src, lds0 + buf * STAGE + (wave * LPW + j) * 1024);
+    }
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // operand pieces: row r of the buffer, elements 16 ks + 8 h .. of the step, at piece r * 8 + ((2 ks + h) ^ (r & 7))
+  unsigned a_row[TM], b_row[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) a_row[i] = wm * (BM / 2) + i * 32 + r32;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) b_row[j] = BM + wn * (BN / 2) + j * 32 + r32;
+
+  const int nk = (K + BK - 1) / BK;
+  const bool tail = K % BK != 0;
+  if (tail && nk == 1) stage_tail(0, 0); else stage(0, 0);
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");      // this wave's pieces of step kt are in LDS
+    __builtin_amdgcn_s_barrier();                             // ... and everyone's; everyone has read step kt - 1
+    if (kt + 1 < nk) {
+      if (tail && kt + 2 == nk) stage_tail((kt + 1) * BK, buf ^ 1);
+      else stage((kt + 1) * BK, buf ^ 1);
+    }
+    const unsigned char* st = lds + buf * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8 a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        a[i] = *(const bf16x8*)(st + (a_row[i] * PCS + ((2 * ks + h) ^ (a_row[i] & 7))) * 16);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        b[j] = *(const bf16x8*)(st + (b_row[j] * PCS + ((2 * ks + h) ^ (b_row[j] & 7))) * 16);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // accumulator 4 q + e of block (i, j): row m0 + wm * 64 + i * 32 + r32, column n0 + wn * (BN / 2) + j * 32 + 8 q + 4 h + e
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const long m = m0 + wm * (BM / 2) + i * 32 + r32;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const long n = n0 + wn * (BN / 2) + j * 32 + q * 8 + h * 4;
+        if (n >= N) continue;                 // (N is a multiple of 4: the four columns are inside or outside together)
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e];
+        if (RESIDUAL) {
+          const bf16x4 r = *(const bf16x4*)(R + m * r_ld + n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += (float)r[e];
+        }
+        bf16x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = static_cast<__bf16>(v[e]);
+        *(bf16x4*)(C + m * c_ld + n) = o;
+      }
+  }
+}
+
+static int g_units = 256;      // compute units of the device: set by whoever knows (the default is an MI355X)
+TIS_EXPORT void tis_gemm_tiles_units(int n) { if (n > 0) g_units = n; }
+
+// W: [N, K] contiguous. R: null, or the residual added to the product; it may be C itself (every element is read and
+// then written by the same lane). Sizes: K and x_ld multiples of 8, N, c_ld and r_ld multiples of 4; X and W 16-byte
+// aligned, C and R 8-byte aligned. Launches only: safe under stream capture.
+TIS_EXPORT int tis_gemm_tiles(const void* X, long x_ld, const void* W, const void* R, long r_ld, void* C, long c_ld,
+                              int M, int N, int K, hipStream_t stream) {
+  if (M < 0 || N < 0 || K < 1) return tis_fail("gemm_tiles: bad size M=%d N=%d K=%d", M, N, K);
+  if (M == 0 || N == 0) return 0;
+  if (K % 8 || x_ld % 8 || x_ld < K) return tis_fail("gemm_tiles: K=%d and the input's row stride %ld must be multiples of 8", K, x_ld);
+  if (N % 4 || c_ld % 4 || c_ld < N || (R && (r_ld % 4 || r_ld < N)))
+    return tis_fail("gemm_tiles: N=%d and the row strides of the output (%ld) and residual (%ld) must be multiples of 4", N, c_ld, r_ld);
+  if (((uintptr_t)X | (uintptr_t)W) % 16 || ((uintptr_t)C | (uintptr_t)R) % 8)
+    return tis_fail("gemm_tiles: inputs must be 16-byte aligned, output and residual 8-byte aligned");
+  if ((long)x_ld * 16 >= (1L << 31) || (long)K * 16 >= (1L << 31)) return tis_fail("gemm_tiles: rows of %ld elements are too long for 32-bit offsets", x_ld);
+  const long tiles_m = (M + GT_BM - 1) / GT_BM;
+  // columns of a tile: 128, or 64 where 128 would leave compute units without a workgroup
+  const bool narrow = tiles_m * ((N + 127) / 128) < g_units;
+  const long tiles = tiles_m * ((N + (narrow ? 63 : 127)) / (narrow ? 64 : 128));
+  if (tiles >= (1L << 31)) return tis_fail("gemm_tiles: %ld tiles are more than a grid holds", tiles);
+#define LAUNCH(BNV, RV)                                                                                    \
+  gemm_tiles_kernel<BNV, RV><<<dim3((unsigned)tiles), GT_WAVES * 64, 0, stream>>>(                         \
+      (const bf16*)X, x_ld, (const bf16*)W, (const bf16*)R, r_ld, (bf16*)C, c_ld, M, N, K)
+  if (narrow) { if (R) LAUNCH(64, true); else LAUNCH(64, false); }
+  else { if (R) LAUNCH(128, true); else LAUNCH(128, false); }
+#undef LAUNCH
+  return tis_launch_status("gemm_tiles");
+}

@@ -38,6 +38,7 @@ SOURCES: Dict[str, str] = {
     "gemm_plain": "gemm_plain.hip",
     "gemm_skinny": "gemm_skinny.hip",
     "gemm_library": "gemm_library.hip",
+    "gemm_tiles": "gemm_tiles.hip",
     "sampling": "sampling.hip",
 }
 HEADERS = ["common.h", "attention_mfma.h"]

@@ -88,6 +88,9 @@ _SIGNATURES["gemm_skinny"] = ("tis_gemm_skinny", {
     "tis_gemm_skinny": [_P, _L, _P, _P, _F, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P],
     "tis_gemm_skinny_qkv_rope": [_P, _L, _P, _P, _F, _P, _L, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
 })
+_SIGNATURES["gemm_tiles"] = ("tis_gemm_tiles", {
+    "tis_gemm_tiles": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _P],
+})
 _SIGNATURES["gemm_library"] = ("tis_gemm_library", {
     "tis_gemm_library_init": [],
     "tis_gemm_library": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _I, _P],
@@ -133,13 +136,16 @@ def library_rows(m: int) -> int:
 
 def product_route(M: int, N: int, K: int, aligned: bool, out_f32: bool, widths, few_rows: int = _FEW_ROWS):
     """Which kernel takes a bfloat16 product of M rows, N output and K input columns: "few_rows" (the fused few-row
-    kernel, in panels of rows beyond its own height), "library" (at library_rows(M) rows) or "plain" (multiply-adds,
-    for operands that do not lie as the other two need them). Pure: the decision can be checked without a device."""
+    kernel, in panels of rows beyond its own height), "library" (at library_rows(M) rows, at the widths of its
+    list), "tiles" (this repository's tiled product, for many rows at any other width) or "plain" (multiply-adds, for
+    operands that do not lie as the others need them). Pure: the decision can be checked without a device."""
     if not aligned:
         return "plain"
-    if M <= few_rows or out_f32 or (N, K) not in widths:
+    if M <= few_rows or out_f32:
         return "few_rows"
-    return "library"
+    if (N, K) in widths:
+        return "library"
+    return "tiles" if N % 4 == 0 else "few_rows"
 
 
 # wavefronts the attention launch aims for, so that short batches still spread over the chip
@@ -491,7 +497,7 @@ class HipOps:
         self.code = _DT[dtype]
         # whatever is not built yet is compiled side by side, not one after the other
         _build.build(["rowwise", "rope_cache", "attention_generic", "gemm_plain", "sampling"] +
-                     (["gemm_skinny", "gemm_library"] if dtype == torch.bfloat16 else []))
+                     (["gemm_skinny", "gemm_library", "gemm_tiles"] if dtype == torch.bfloat16 else []))
         self.rowwise = library("rowwise")
         self.rope = library("rope_cache")
         self.attn_generic = library("attention_generic")
@@ -506,6 +512,8 @@ class HipOps:
         self.units = int(torch.cuda.get_device_properties(self.device).multi_processor_count) or _CHIP_UNITS
         if dtype == torch.bfloat16:
             self.gemm_skinny.cdll.tis_gemm_skinny_units(self.units)
+            self.gemm_tiles = library("gemm_tiles")
+            self.gemm_tiles.cdll.tis_gemm_tiles_units(self.units)
             self.gemm_library = library("gemm_library")
             with torch.cuda.device(self.device):
                 self.gemm_library.tis_gemm_library_init()
@@ -715,6 +723,12 @@ class HipOps:
             x = self.rmsnorm(x, rms[0], rms[1])
         if route == "library":
             return self._linear_library(x, w, residual)
+        if route == "tiles":
+            out = self.empty(M, N)
+            self.gemm_tiles.tis_gemm_tiles(_ptr(x), x.stride(0), _ptr(w), _ptr(residual),
+                                           residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0),
+                                           M, N, K, self._stream())
+            return out
         out = self.empty(M, N, dtype=out_dtype)
         self.gemm_plain.tis_gemm_plain(1, _DT[out_dtype], _ptr(x), x.stride(0), _ptr(w), K, _ptr(residual),
                                        residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0), M, N,
@@ -727,6 +741,8 @@ class HipOps:
         aligned = K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
         route = product_route(M, N, K, aligned, out_dtype == torch.float32, self.library_widths, self.few_rows)
         if route == "library" and residual is not None and (residual.stride(0) % 8 or residual.data_ptr() % 16):
+            route = "few_rows"
+        if route == "tiles" and residual is not None and (residual.stride(0) % 4 or residual.data_ptr() % 8):
             route = "few_rows"
         if route == "few_rows" and M > 8 * self.few_rows and (N, K) not in self._warned_widths \
                 and out_dtype != torch.float32:

@@ -7,9 +7,11 @@
 // A workgroup of four waves (2 x 2) owns a tile of 128 rows x 128 or 64 columns and walks K in steps of 64. A step's
 // operand rows, 128 bytes each, are copied into LDS by global_load_lds_dwordx4 (no registers; eight lanes read one
 // row's 128 bytes), one step ahead of the products, into one of two buffers; two workgroups share a compute unit and
-// fill each other's waits. A row's eight 16-byte pieces lie in LDS with their index XORed by the row's number, so
-// that the 32 rows an operand fetch reads for one piece index fall into different banks; the copying lane picks the
-// piece that belongs in its slot. The result tile is computed transposed (W's rows are the first operand), so that a
+// fill each other's waits. A row's eight 16-byte pieces lie in LDS with their index XORed by half the row's number:
+// an operand fetch reads one piece index of 32 rows, LDS serves sixteen lanes at a time, and sixteen rows of 128
+// bytes are eight such indices at each of two offsets in the 256 bytes that the banks span, so no two of them meet
+// (XORed by the row's number itself, rows r and r + 8 did: half of the LDS's busy cycles were bank conflicts). The
+// copying lane picks the piece that belongs in its slot. The result tile is computed transposed (W's rows are the first operand), so that a
 // lane ends up with four consecutive columns of one row: 8-byte stores, and the residual read the same way.
 // A row's sums run over K in the same order whatever M is: its result does not depend on the other rows.
 #include "common.h"
@@ -60,24 +62,22 @@ __global__ __launch_bounds__(GT_WAVES * 64) void gemm_tiles_kernel(
   const unsigned lds0 = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds;
 
   // The wave's loads of a step: load j brings rows 8 (wave * LPW + j) .. +7 of the buffer, lane (row, slot) the piece
-  // slot ^ (row & 7) of its row. Rows past the matrix's last are the last row again (their results are not stored).
+  // slot ^ ((row >> 1) & 7) of its row. Rows past the matrix's last are the last row again (their results are not
+  // stored).
   const unsigned char* first_row[LPW];       // of the load's first row, at K offset 0 (the same on all lanes)
   unsigned lane_off[LPW];                    // the lane's piece from there, in bytes
-  int lane_piece;                            // which 8 elements of a step's 64 the lane brings
-  {
-    const int slot = lane & 7;
-    lane_piece = slot ^ ((lane >> 3) & 7);   // (a load's first row is a multiple of 8)
-  }
+  int lane_piece[LPW];                       // which 8 elements of a step's 64 the lane brings
 #pragma unroll
   for (int j = 0; j < LPW; ++j) {
     const int row0 = (wave * LPW + j) * 8, row = row0 + (lane >> 3);
+    lane_piece[j] = (lane & 7) ^ ((row >> 1) & 7);
     const bool of_x = row0 < BM;
     const long ld = of_x ? x_ld : (long)K;
     const long last = of_x ? (long)M - 1 : (long)N - 1;
     const long g_first = min(last, of_x ? m0 + row0 : n0 + (row0 - BM));
     const long g_row = min(last, of_x ? m0 + row : n0 + (row - BM));
     first_row[j] = (const unsigned char*)(of_x ? X : W) + g_first * ld * 2;
-    lane_off[j] = (unsigned)((g_row - g_first) * ld * 2 + lane_piece * 16);
+    lane_off[j] = (unsigned)((g_row - g_first) * ld * 2 + lane_piece[j] * 16);
   }
   auto stage = [&](int k0, int buf) {
 #pragma unroll
@@ -86,9 +86,9 @@ __global__ __launch_bounds__(GT_WAVES * 64) void gemm_tiles_kernel(
   };
   // the last step of a K that is no multiple of 64: pieces past the end come from a block of zeros
   auto stage_tail = [&](int k0, int buf) {
-    const bool inside = k0 + lane_piece * 8 < K;
 #pragma unroll
     for (int j = 0; j < LPW; ++j) {
+      const bool inside = k0 + lane_piece[j] * 8 < K;
       const unsigned char* src = inside ? first_row[j] + (long)k0 * 2 + lane_off[j] : gt_zeros;
       gt_copy16(src, lds0 + buf * STAGE + (wave * LPW + j) * 1024);
     }
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(GT_WAVES * 64) void gemm_tiles_kernel(
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // operand pieces: row r of the buffer, elements 16 ks + 8 h .. of the step, at piece r * 8 + ((2 ks + h) ^ (r & 7))
+  // operand pieces: row r of the buffer, elements 16 ks + 8 h .. of the step, at piece r * 8 + ((2 ks + h) ^ ((r >> 1) & 7))
   unsigned a_row[TM], b_row[TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i) a_row[i] = wm * (BM / 2) + i * 32 + r32;
@@ -126,10 +126,10 @@ __global__ __launch_bounds__(GT_WAVES * 64) void gemm_tiles_kernel(
       bf16x8 a[TM], b[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        a[i] = *(const bf16x8*)(st + (a_row[i] * PCS + ((2 * ks + h) ^ (a_row[i] & 7))) * 16);
+        a[i] = *(const bf16x8*)(st + (a_row[i] * PCS + ((2 * ks + h) ^ ((a_row[i] >> 1) & 7))) * 16);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        b[j] = *(const bf16x8*)(st + (b_row[j] * PCS + ((2 * ks + h) ^ (b_row[j] & 7))) * 16);
+        b[j] = *(const bf16x8*)(st + (b_row[j] * PCS + ((2 * ks + h) ^ ((b_row[j] >> 1) & 7))) * 16);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll

@@ -642,11 +642,11 @@ def test_product_with_norm_residual_and_gate_for_many_rows(ops_for, M, N, K):
 
 
 @pytest.mark.parametrize("M", [129, 200, 777, 2049])
-@pytest.mark.parametrize("N,K", [(64, 8), (132, 72), (520, 1528), (1536, 640), (4096, 4096), (6148, 200)])
+@pytest.mark.parametrize("N,K", [(64, 8), (132, 72), (520, 1528), (1536, 640), (4096, 4096), (6148, 200), (8196, 264)])
 def test_tiled_product_at_widths_the_library_is_not_used_at(ops_for, M, N, K):
     """Many rows at a width outside the library's list go to the tiled product of this repository: row and column
-    counts that end inside a tile, a K that ends inside a step of 64 (down to a single piece of 8), tiles of 64 and of
-    128 columns, with a residual that is the output itself or another tensor. Against exact sums of the same bfloat16
+    counts that end inside a tile, a K that ends inside a step of 64 (down to a single piece of 8), tiles of 64, 128
+    and (2,049 rows by 8,196 columns) 256 columns, with a residual that is the output itself or another tensor. Against exact sums of the same bfloat16
     operands; and a row's result does not depend on which tile or rows it shares."""
     from tiny_inference_server_amd.ops.hip_ops import product_route
     ops = ops_for(torch.bfloat16)

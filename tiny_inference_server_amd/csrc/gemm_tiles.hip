@@ -4,7 +4,8 @@
 // PFLOP/s at 2,048 rows. This kernel reaches 0.45 to 0.95 on the same shapes; the library's kernels, where they may be
 // used, 0.5 to 1.3.) The reference's engine uses a library product here (x @ W, main_models_new.py:19-20).
 //
-// A workgroup of four waves (2 x 2) owns a tile of 128 rows x 128 or 64 columns and walks K in steps of 64. A step's
+// A workgroup of four waves (2 x 2) owns a tile of 128 rows x 128 or 64 columns, or one of eight waves (2 x 4) a tile
+// of 256 x 256 where that still gives every compute unit a workgroup, and walks K in steps of 64. A step's
 // operand rows, 128 bytes each, are copied into LDS by global_load_lds_dwordx4 (no registers; eight lanes read one
 // row's 128 bytes), one step ahead of the products, into one of two buffers; two workgroups share a compute unit and
 // fill each other's waits. A row's eight 16-byte pieces lie in LDS with their index XORed by half the row's number:
@@ -22,7 +23,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-static constexpr int GT_BM = 128, GT_BK = 64, GT_WAVES = 4, GT_PIECES = GT_BK / 8;
+static constexpr int GT_BK = 64, GT_PIECES = GT_BK / 8;
 
 // what lanes past the end of K read in the last step: zeros
 static __device__ __attribute__((aligned(16))) unsigned char gt_zeros[16];
@@ -45,18 +46,19 @@ __device__ __forceinline__ void gt_copy16(const void* lane_src, unsigned lds_add
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(lane_src), "s"(base) : "memory", "m0");
 }
 
-template <int BN, bool RESIDUAL>
-__global__ __launch_bounds__(GT_WAVES * 64) void gemm_tiles_kernel(
+// BM x BN: the workgroup's tile; WM x WN: its waves, each with (BM / WM) x (BN / WN) of it
+template <int BM, int BN, int WM, int WN, bool RESIDUAL>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_tiles_kernel(
     const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const bf16* R, long r_ld, bf16* C, long c_ld,
     int M, int N, int K) {
-  constexpr int BM = GT_BM, BK = GT_BK, PCS = GT_PIECES, ROWS = BM + BN;
+  constexpr int BK = GT_BK, PCS = GT_PIECES, ROWS = BM + BN, GT_WAVES = WM * WN;
   constexpr int STAGE = ROWS * BK * 2;                  // bytes of a buffer: X's rows, then W's
   constexpr int LPW = ROWS * PCS / 64 / GT_WAVES;       // loads of a step that each wave issues, 8 rows each
-  constexpr int TM = BM / 2 / 32, TN = BN / 2 / 32;     // 32 x 32 result tiles of a wave
-  static_assert(ROWS * PCS % (64 * GT_WAVES) == 0 && TN >= 1, "tile sizes");
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;   // 32 x 32 result tiles of a wave
+  static_assert(ROWS * PCS % (64 * GT_WAVES) == 0 && TM >= 1 && TN >= 1 && 2 * STAGE <= 160 * 1024, "tile sizes");
   __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * STAGE];
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, r32 = lane & 31, h = lane >> 5;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   const int tiles_m = (M + BM - 1) / BM;
   const long m0 = (long)(blockIdx.x % tiles_m) * BM, n0 = (long)(blockIdx.x / tiles_m) * BN;
   const unsigned lds0 = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds;
@@ -105,9 +107,9 @@ __global__ __launch_bounds__(GT_WAVES * 64) void gemm_tiles_kernel(
   // operand pieces: row r of the buffer, elements 16 ks + 8 h .. of the step, at piece r * 8 + ((2 ks + h) ^ ((r >> 1) & 7))
   unsigned a_row[TM], b_row[TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i) a_row[i] = wm * (BM / 2) + i * 32 + r32;
+  for (int i = 0; i < TM; ++i) a_row[i] = wm * (BM / WM) + i * 32 + r32;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) b_row[j] = BM + wn * (BN / 2) + j * 32 + r32;
+  for (int j = 0; j < TN; ++j) b_row[j] = BM + wn * (BN / WN) + j * 32 + r32;
 
   const int nk = (K + BK - 1) / BK;
   const bool tail = K % BK != 0;
@@ -138,16 +140,16 @@ __global__ __launch_bounds__(GT_WAVES * 64) void gemm_tiles_kernel(
     }
   }
 
-  // accumulator 4 q + e of block (i, j): row m0 + wm * 64 + i * 32 + r32, column n0 + wn * (BN / 2) + j * 32 + 8 q + 4 h + e
+  // accumulator 4 q + e of block (i, j): row m0 + wm * (BM / WM) + i * 32 + r32, column n0 + wn * (BN / WN) + j * 32 + 8 q + 4 h + e
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const long m = m0 + wm * (BM / 2) + i * 32 + r32;
+    const long m = m0 + wm * (BM / WM) + i * 32 + r32;
     if (m >= M) continue;
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const long n = n0 + wn * (BN / 2) + j * 32 + q * 8 + h * 4;
+        const long n = n0 + wn * (BN / WN) + j * 32 + q * 8 + h * 4;
         if (n >= N) continue;                 // (N is a multiple of 4: the four columns are inside or outside together)
         float v[4];
 #pragma unroll
@@ -181,16 +183,19 @@ TIS_EXPORT int tis_gemm_tiles(const void* X, long x_ld, const void* W, const voi
   if (((uintptr_t)X | (uintptr_t)W) % 16 || ((uintptr_t)C | (uintptr_t)R) % 8)
     return tis_fail("gemm_tiles: inputs must be 16-byte aligned, output and residual 8-byte aligned");
   if ((long)x_ld * 16 >= (1L << 31) || (long)K * 16 >= (1L << 31)) return tis_fail("gemm_tiles: rows of %ld elements are too long for 32-bit offsets", x_ld);
-  const long tiles_m = (M + GT_BM - 1) / GT_BM;
-  // columns of a tile: 128, or 64 where 128 would leave compute units without a workgroup
-  const bool narrow = tiles_m * ((N + 127) / 128) < g_units;
-  const long tiles = tiles_m * ((N + (narrow ? 63 : 127)) / (narrow ? 64 : 128));
+  // The tile: 256 x 256 on eight waves where that gives every compute unit a workgroup (it moves half the bytes into
+  // LDS per product that 128 x 128 does: 2,048 x 8,192 x 1,536 at 0.92 instead of 0.84 PFLOP/s); else 128 x 128 on
+  // four; 128 x 64 where 128 x 128 would leave compute units without a workgroup.
+  const long big = (long)((M + 255) / 256) * ((N + 255) / 256), mid = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const int bm = big >= g_units ? 256 : 128, bn = big >= g_units ? 256 : mid >= g_units ? 128 : 64;
+  const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
   if (tiles >= (1L << 31)) return tis_fail("gemm_tiles: %ld tiles are more than a grid holds", tiles);
-#define LAUNCH(BNV, RV)                                                                                    \
-  gemm_tiles_kernel<BNV, RV><<<dim3((unsigned)tiles), GT_WAVES * 64, 0, stream>>>(                         \
+#define LAUNCH(BMV, BNV, WMV, WNV, RV)                                                                     \
+  gemm_tiles_kernel<BMV, BNV, WMV, WNV, RV><<<dim3((unsigned)tiles), WMV * WNV * 64, 0, stream>>>(         \
       (const bf16*)X, x_ld, (const bf16*)W, (const bf16*)R, r_ld, (bf16*)C, c_ld, M, N, K)
-  if (narrow) { if (R) LAUNCH(64, true); else LAUNCH(64, false); }
-  else { if (R) LAUNCH(128, true); else LAUNCH(128, false); }
+  if (bm == 256) { if (R) LAUNCH(256, 256, 2, 4, true); else LAUNCH(256, 256, 2, 4, false); }
+  else if (bn == 128) { if (R) LAUNCH(128, 128, 2, 2, true); else LAUNCH(128, 128, 2, 2, false); }
+  else { if (R) LAUNCH(128, 64, 2, 2, true); else LAUNCH(128, 64, 2, 2, false); }
 #undef LAUNCH
   return tis_launch_status("gemm_tiles");
 }

@@ -214,46 +214,47 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
     rows at 1,000 beside 8 decoded tokens at 4,095: 54.9 / 64.7, one of 256 rows 40.6 / 30.1, one of 128 35.9 / 23.9.
     """
     none = np.zeros((0, 2), dtype=np.int32)
-    single = all(n <= 1 for _, _, n in seq_rows)
-    if single:
+    # (arrays over all requests at once: a step may hold hundreds, and this runs for every stage of every step that
+    # is not replayed from a graph)
+    rows = np.asarray(seq_rows, dtype=np.int64).reshape(-1, 3)
+    first, p0, n = rows[:, 0], rows[:, 1], rows[:, 2]
+    if not (n > 1).any():
         nb = 1
         while group_size > 16 * nb:
             nb *= 2
-        return nb, np.asarray([(first, 1) for first, _, n in seq_rows if n], dtype=np.int32).reshape(-1, 2), none, (0, 0)
-    tile_rows = _ATTN_TILE_WAVES * (tile_cols // group_size)
-    tiled = [(f, p0, n) for f, p0, n in seq_rows if tile_rows and n >= max(2, tile_rows // 2)]
-    if tiled and n_kv_heads:
-        work = sum(int(((p0 + np.minimum(np.arange(0, n, tile_rows) + tile_rows, n) + 31) // 32).sum())
-                   for _, p0, n in tiled) * n_kv_heads
-        deep = any(n == 1 and p0 >= 512 for _, p0, n in seq_rows)
-        if deep and work < _ATTN_TILE_MIN_WORK_MIXED:
-            tiled = []
-    taken = {f for f, _, _ in tiled}
-    rest = [(f, p0, n) for f, p0, n in seq_rows if n > 0 and f not in taken]
+        live = n > 0
+        return nb, np.stack((first[live], n[live]), axis=1).astype(np.int32), none, (0, 0)
 
-    def cut(segments, per_item):
-        if not segments:
+    def cut(which, per_item):
+        if not which.any():
             return none, (0, 0)
-        first, p0, n = np.asarray(segments, dtype=np.int64).reshape(-1, 3).T
-        k = -(-n // per_item)                                          # items of each segment
+        f, q0, m = first[which], p0[which], n[which]
+        k = -(-m // per_item)                                          # items of each segment
         r = (np.arange(int(k.sum())) - np.repeat(np.cumsum(k) - k, k)) * per_item    # an item's first row in its segment
-        counts = np.minimum(per_item, np.repeat(n, k) - r)
-        firsts = np.repeat(first, k) + r
-        keys = np.repeat(p0, k) + r + counts
+        counts = np.minimum(per_item, np.repeat(m, k) - r)
+        firsts = np.repeat(f, k) + r
+        keys = np.repeat(q0, k) + r + counts
         # those with the most keys first: under a causal mask the last rows of a prompt are the longest, and
         # started last they would run on alone while the rest of the chip idles
         order = np.argsort(-keys, kind="stable")
         steps = (keys + 31) // 32
         return np.stack((firsts[order], counts[order]), axis=1).astype(np.int32), (int(steps.sum()), int(steps.max()))
 
+    tile_rows = _ATTN_TILE_WAVES * (tile_cols // group_size)
+    tiled = (n >= max(2, tile_rows // 2)) if tile_rows else np.zeros(len(n), dtype=bool)
+    tiles, steps = cut(tiled, tile_rows) if tile_rows else (none, (0, 0))
+    if len(tiles) and n_kv_heads and steps[0] * n_kv_heads < _ATTN_TILE_MIN_WORK_MIXED \
+            and ((n == 1) & (p0 >= 512)).any():
+        # beside decoded tokens deep in their requests: too little work for tiles
+        tiled, tiles, steps = np.zeros(len(n), dtype=bool), none, (0, 0)
+    rest = (n > 0) & ~tiled
     nb = 2
     # 64-column items halve what a portion reads of its keys and values; they pay once there are enough of them
     # to fill the chip, and cost where a few long chains of steps set the time
-    if group_size <= 64 and sum(-(-n // max(1, 64 // group_size)) for _, _, n in rest) >= 384:
+    if group_size <= 64 and int((-(-n[rest] // max(1, 64 // group_size))).sum()) >= 384:
         nb = 4
     while group_size > 16 * nb:
         nb *= 2
-    tiles, steps = cut(tiled, tile_rows)
     return nb, cut(rest, max(1, (16 * nb) // group_size))[0], tiles, steps
 
 

@@ -660,9 +660,13 @@ def test_tiled_product_at_widths_the_library_is_not_used_at(ops_for, M, N, K):
     torch.testing.assert_close(ops.linear(x.cuda(), w.cuda(), residual=res.cuda()).cpu().double(), want + res.double(), **t)
     # the residual as the output's own memory
     out, xd, wd = res.clone().cuda(), x.cuda(), w.cuda()
-    ops.gemm_tiles.tis_gemm_tiles(xd.data_ptr(), K, wd.data_ptr(), out.data_ptr(), N, out.data_ptr(), N, M, N, K,
+    ops.gemm_tiles.tis_gemm_tiles(xd.data_ptr(), K, wd.data_ptr(), out.data_ptr(), N, out.data_ptr(), N, M, N, K, 0,
                                   ops._stream())
     torch.testing.assert_close(out.cpu().double(), want + res.double(), **t)
+    # 32-bit results (the output table's logits for many rows): the sums as they are
+    lg = ops.linear(xd, wd, out_dtype=torch.float32)
+    assert lg.dtype == torch.float32
+    torch.testing.assert_close(lg.cpu().double(), want, rtol=1e-4, atol=1e-4)
     # a row moved to another place among other rows gives the same bits
     others = rnd((M, K), torch.bfloat16, 63, 2.0)
     others[M - 1] = x[3]

@@ -64,7 +64,8 @@ def test_routes():
     assert product_route(65, 2304, 1536, True, False, w, few_rows=64) == "library"
     assert product_route(hip_ops._FEW_ROWS, 2304, 1536, True, False, w) == "few_rows"
     assert product_route(hip_ops._FEW_ROWS + 1, 2304, 1536, True, False, w) == "library"
-    assert product_route(2048, 2304, 1536, True, True, w) == "few_rows"         # 32-bit results: own kernels
+    assert product_route(2048, 2304, 1536, True, True, w) == "tiles"            # 32-bit results: own kernels
+    assert product_route(100, 2304, 1536, True, True, w) == "few_rows"
     assert product_route(2048, 6144, 4096, True, False, w) == "tiles"           # a width nobody listed: own kernel
     assert product_route(128, 6144, 4096, True, False, w) == "few_rows"
     assert product_route(2048, 6146, 4096, True, False, w) == "few_rows"        # ... whose stores need N in steps of 4
@@ -117,8 +118,8 @@ def test_no_unlisted_width_and_no_unrounded_row_count_reaches_the_library(seed):
             assert X % 16 == 0 and W % 16 == 0 and C % 16 == 0 and R % 16 == 0
             assert x_ld >= K and c_ld >= N
         elif fn == "tis_gemm_tiles":
-            X, x_ld, W, R, r_ld, C, c_ld, rows, n, k = a[:10]
-            assert (rows, n, k) == (M, N, K) and (N, K) not in library_widths() and M > ops.few_rows
+            X, x_ld, W, R, r_ld, C, c_ld, rows, n, k, f32 = a[:11]
+            assert (rows, n, k) == (M, N, K) and (N, K) not in library_widths() and M > ops.few_rows and f32 == 0
             assert K % 8 == 0 and N % 4 == 0 and X % 16 == 0 and W % 16 == 0 and C % 8 == 0 and R % 8 == 0
             assert C == out.data_ptr() and inside(out, C, M, c_ld, N) and x_ld >= K
         else:

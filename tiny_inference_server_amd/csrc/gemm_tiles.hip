@@ -22,6 +22,7 @@ TIS_DEFINE_LAST_ERROR(tis_gemm_tiles)
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 static constexpr int GT_BK = 64, GT_PIECES = GT_BK / 8;
 
@@ -47,9 +48,9 @@ __device__ __forceinline__ void gt_copy16(const void* lane_src, unsigned lds_add
 }
 
 // BM x BN: the workgroup's tile; WM x WN: its waves, each with (BM / WM) x (BN / WN) of it
-template <int BM, int BN, int WM, int WN, bool RESIDUAL>
+template <int BM, int BN, int WM, int WN, bool RESIDUAL, typename TO>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_tiles_kernel(
-    const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const bf16* R, long r_ld, bf16* C, long c_ld,
+    const bf16* __restrict__ X, long x_ld, const bf16* __restrict__ W, const bf16* R, long r_ld, TO* C, long c_ld,
     int M, int N, int K) {
   constexpr int BK = GT_BK, PCS = GT_PIECES, ROWS = BM + BN, GT_WAVES = WM * WN;
   constexpr int STAGE = ROWS * BK * 2;                  // bytes of a buffer: X's rows, then W's
@@ -159,10 +160,14 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tiles_kernel(
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] += (float)r[e];
         }
-        bf16x4 o;
+        if constexpr (sizeof(TO) == 4) {
+          *(f32x4*)(C + m * c_ld + n) = (f32x4){v[0], v[1], v[2], v[3]};       // the 32-bit sums as they are
+        } else {
+          bf16x4 o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = static_cast<__bf16>(v[e]);
-        *(bf16x4*)(C + m * c_ld + n) = o;
+          for (int e = 0; e < 4; ++e) o[e] = static_cast<__bf16>(v[e]);
+          *(bf16x4*)(C + m * c_ld + n) = o;
+        }
       }
   }
 }
@@ -170,18 +175,20 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tiles_kernel(
 static int g_units = 256;      // compute units of the device: set by whoever knows (the default is an MI355X)
 TIS_EXPORT void tis_gemm_tiles_units(int n) { if (n > 0) g_units = n; }
 
-// W: [N, K] contiguous. R: null, or the residual added to the product; it may be C itself (every element is read and
-// then written by the same lane). Sizes: K and x_ld multiples of 8, N, c_ld and r_ld multiples of 4; X and W 16-byte
-// aligned, C and R 8-byte aligned. Launches only: safe under stream capture.
+// W: [N, K] contiguous. R: null, or the residual (bfloat16) added to the product; it may be C itself (every element is
+// read and then written by the same lane). out_f32: C holds 32-bit floats, the sums as they are (the output table's
+// logits), and takes no residual. Sizes: K and x_ld multiples of 8, N, c_ld and r_ld multiples of 4; X and W 16-byte
+// aligned, C and R 8-byte aligned (a 32-bit C 16-byte). Launches only: safe under stream capture.
 TIS_EXPORT int tis_gemm_tiles(const void* X, long x_ld, const void* W, const void* R, long r_ld, void* C, long c_ld,
-                              int M, int N, int K, hipStream_t stream) {
+                              int M, int N, int K, int out_f32, hipStream_t stream) {
   if (M < 0 || N < 0 || K < 1) return tis_fail("gemm_tiles: bad size M=%d N=%d K=%d", M, N, K);
   if (M == 0 || N == 0) return 0;
   if (K % 8 || x_ld % 8 || x_ld < K) return tis_fail("gemm_tiles: K=%d and the input's row stride %ld must be multiples of 8", K, x_ld);
   if (N % 4 || c_ld % 4 || c_ld < N || (R && (r_ld % 4 || r_ld < N)))
     return tis_fail("gemm_tiles: N=%d and the row strides of the output (%ld) and residual (%ld) must be multiples of 4", N, c_ld, r_ld);
-  if (((uintptr_t)X | (uintptr_t)W) % 16 || ((uintptr_t)C | (uintptr_t)R) % 8)
-    return tis_fail("gemm_tiles: inputs must be 16-byte aligned, output and residual 8-byte aligned");
+  if (((uintptr_t)X | (uintptr_t)W) % 16 || ((uintptr_t)C | (uintptr_t)R) % 8 || (out_f32 && (uintptr_t)C % 16))
+    return tis_fail("gemm_tiles: inputs must be 16-byte aligned, output and residual 8-byte aligned (a 32-bit output 16-byte)");
+  if (out_f32 && R) return tis_fail("gemm_tiles: a 32-bit result takes no residual");
   if ((long)x_ld * 16 >= (1L << 31) || (long)K * 16 >= (1L << 31)) return tis_fail("gemm_tiles: rows of %ld elements are too long for 32-bit offsets", x_ld);
   // The tile: 256 x 256 on eight waves where that gives every compute unit a workgroup (it moves half the bytes into
   // LDS per product that 128 x 128 does: 2,048 x 8,192 x 1,536 at 0.92 instead of 0.84 PFLOP/s); else 128 x 128 on
@@ -190,12 +197,19 @@ TIS_EXPORT int tis_gemm_tiles(const void* X, long x_ld, const void* W, const voi
   const int bm = big >= g_units ? 256 : 128, bn = big >= g_units ? 256 : mid >= g_units ? 128 : 64;
   const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
   if (tiles >= (1L << 31)) return tis_fail("gemm_tiles: %ld tiles are more than a grid holds", tiles);
-#define LAUNCH(BMV, BNV, WMV, WNV, RV)                                                                     \
-  gemm_tiles_kernel<BMV, BNV, WMV, WNV, RV><<<dim3((unsigned)tiles), WMV * WNV * 64, 0, stream>>>(         \
-      (const bf16*)X, x_ld, (const bf16*)W, (const bf16*)R, r_ld, (bf16*)C, c_ld, M, N, K)
-  if (bm == 256) { if (R) LAUNCH(256, 256, 2, 4, true); else LAUNCH(256, 256, 2, 4, false); }
-  else if (bn == 128) { if (R) LAUNCH(128, 128, 2, 2, true); else LAUNCH(128, 128, 2, 2, false); }
-  else { if (R) LAUNCH(128, 64, 2, 2, true); else LAUNCH(128, 64, 2, 2, false); }
+#define LAUNCH(BMV, BNV, WMV, WNV, RV, TOV)                                                                \
+  gemm_tiles_kernel<BMV, BNV, WMV, WNV, RV, TOV><<<dim3((unsigned)tiles), WMV * WNV * 64, 0, stream>>>(    \
+      (const bf16*)X, x_ld, (const bf16*)W, (const bf16*)R, r_ld, (TOV*)C, c_ld, M, N, K)
+#define PICK(BMV, BNV, WMV, WNV)                                \
+  {                                                             \
+    if (out_f32) LAUNCH(BMV, BNV, WMV, WNV, false, float);      \
+    else if (R) LAUNCH(BMV, BNV, WMV, WNV, true, bf16);         \
+    else LAUNCH(BMV, BNV, WMV, WNV, false, bf16);               \
+  }
+  if (bm == 256) PICK(256, 256, 2, 4)
+  else if (bn == 128) PICK(128, 128, 2, 2)
+  else PICK(128, 64, 2, 2)
+#undef PICK
 #undef LAUNCH
   return tis_launch_status("gemm_tiles");
 }

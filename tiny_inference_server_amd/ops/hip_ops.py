@@ -89,7 +89,7 @@ _SIGNATURES["gemm_skinny"] = ("tis_gemm_skinny", {
     "tis_gemm_skinny_qkv_rope": [_P, _L, _P, _P, _F, _P, _L, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
 })
 _SIGNATURES["gemm_tiles"] = ("tis_gemm_tiles", {
-    "tis_gemm_tiles": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _P],
+    "tis_gemm_tiles": [_P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _I, _P],
 })
 _SIGNATURES["gemm_library"] = ("tis_gemm_library", {
     "tis_gemm_library_init": [],
@@ -137,13 +137,13 @@ def library_rows(m: int) -> int:
 def product_route(M: int, N: int, K: int, aligned: bool, out_f32: bool, widths, few_rows: int = _FEW_ROWS):
     """Which kernel takes a bfloat16 product of M rows, N output and K input columns: "few_rows" (the fused few-row
     kernel, in panels of rows beyond its own height), "library" (at library_rows(M) rows, at the widths of its
-    list), "tiles" (this repository's tiled product, for many rows at any other width) or "plain" (multiply-adds, for
-    operands that do not lie as the others need them). Pure: the decision can be checked without a device."""
+    list), "tiles" (this repository's tiled product, for many rows at any other width and for 32-bit results at any
+    width) or "plain" (multiply-adds, for operands that do not lie as the others need them). Pure: the decision can be checked without a device."""
     if not aligned:
         return "plain"
-    if M <= few_rows or out_f32:
+    if M <= few_rows:
         return "few_rows"
-    if (N, K) in widths:
+    if (N, K) in widths and not out_f32:
         return "library"
     return "tiles" if N % 4 == 0 else "few_rows"
 
@@ -725,10 +725,12 @@ class HipOps:
         if route == "library":
             return self._linear_library(x, w, residual)
         if route == "tiles":
-            out = self.empty(M, N)
+            if out_dtype == torch.float32 and residual is not None:
+                raise KernelError("linear: a 32-bit result of bfloat16 operands takes no residual")
+            out = self.empty(M, N, dtype=out_dtype)
             self.gemm_tiles.tis_gemm_tiles(_ptr(x), x.stride(0), _ptr(w), _ptr(residual),
                                            residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0),
-                                           M, N, K, self._stream())
+                                           M, N, K, 1 if out_dtype == torch.float32 else 0, self._stream())
             return out
         out = self.empty(M, N, dtype=out_dtype)
         self.gemm_plain.tis_gemm_plain(1, _DT[out_dtype], _ptr(x), x.stride(0), _ptr(w), K, _ptr(residual),

@@ -642,7 +642,7 @@ def test_product_with_norm_residual_and_gate_for_many_rows(ops_for, M, N, K):
 
 
 @pytest.mark.parametrize("M", [129, 200, 777, 2049])
-@pytest.mark.parametrize("N,K", [(64, 8), (132, 72), (520, 1528), (1536, 640), (4096, 4096), (6148, 200), (8196, 264)])
+@pytest.mark.parametrize("N,K", [(4, 16), (64, 8), (132, 72), (520, 1528), (1536, 640), (4096, 4096), (6148, 200), (8196, 264)])
 def test_tiled_product_at_widths_the_library_is_not_used_at(ops_for, M, N, K):
     """Many rows at a width outside the library's list go to the tiled product of this repository: row and column
     counts that end inside a tile, a K that ends inside a step of 64 (down to a single piece of 8), tiles of 64, 128

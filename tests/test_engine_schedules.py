@@ -193,6 +193,49 @@ def test_random_schedules(name, dtype, backend, seed):
     assert eng.free_pages() == eng.total_pages()
 
 
+def drawn_configuration(seed):
+    """A tiny configuration with every size drawn: heads and groups (also groups that do not divide a wave's columns),
+    head sizes in steps of 8 (those in steps of 16 run on the matrix cores, the others on the general kernel), widths
+    and vocabularies that are no power of two, layers, prediction heads, the norms' eps, the rotary base, the page."""
+    import random
+    from tiny_inference_server_amd.config import GqaMtpConfig
+    rng = random.Random(1000 + seed)
+    n_kv, group = rng.choice([1, 1, 2, 3, 4]), rng.choice([1, 2, 3, 4, 5, 8])
+    hd = rng.choice([16, 32, 48, 64, 80, 96, 128, 8, 24, 40])
+    while n_kv * group * hd > 1280:
+        n_kv, group = max(1, n_kv - 1), max(1, group - 1)
+    cfg = GqaMtpConfig(d_model=n_kv * group * hd, vocab_size=rng.choice([97, 300, 515, 1000, 2049, 3001]),
+                       max_context=rng.choice([200, 320, 512]), rope_base=rng.choice([1000.0, 10000.0, 500000.0]),
+                       n_heads=n_kv * group, n_layers=rng.randint(1, 3),
+                       ffn_hidden=rng.choice([88, 176, 200, 264, 320, 520, 1000, 1408]), group_size=group,
+                       mtp_heads=rng.randint(0, 2), rms_eps=rng.choice([2e-8, 1e-6, 1e-5]),
+                       tie_embeddings=rng.random() < 0.5)
+    wide = dict(std=0.02, sharpen=2.0) if cfg.d_model >= 512 else {}
+    return rng, dict(cfg=cfg, page_size=rng.choice([8, 16, 16, 32]), gain_jitter=0.1, seed=100 + seed, **wide)
+
+
+@pytest.mark.parametrize("seed,backend", [pytest.param(s, "hip", marks=pytest.mark.gpu) for s in range(24)]
+                         + [(s, "torch") for s in (0, 3, 29)])
+def test_drawn_configurations_under_drawn_schedules(seed, backend):
+    """Not the few configurations the other tests know: every size of the model drawn at random, then a precision and
+    a family of schedules drawn too, against the plain implementation at the fixed tolerances."""
+    name = f"drawn{seed}"
+    rng, H.TINY[name] = drawn_configuration(seed)
+    cfg = H.TINY[name]["cfg"]
+    dtype = rng.choice(["bfloat16", "bfloat16", "float32"])
+    kind = rng.choice(["whole", "tail", "portions", "mixed", "mixed"])
+    lengths = [rng.randint(1, min(150, cfg.max_context - 4)) for _ in range(rng.randint(2, 7))]
+    reqs = requests_for(name, lengths, seed=seed)
+    steps, peak = {"whole": lambda: (H.whole_trace(reqs), 256), "tail": lambda: (H.tail_decode_trace(reqs, 32), 256),
+                   "portions": lambda: (H.portions_trace(reqs, seed=seed), 256),
+                   "mixed": lambda: H.mixed_trace(reqs, max_live=4, seed=seed)}[kind]()
+    folder, eng = make_engine(name, dtype, backend, max_tokens=max(peak, 64))
+    main, heads = H.run_trace(eng, steps)
+    H.compare_with_plain(folder, reqs, main, heads, TOL[dtype] * scale_of(folder, reqs), cfg.mtp_heads, steps)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()
+
+
 @pytest.mark.parametrize("backend", backends())
 @pytest.mark.parametrize("name,dtype", [("D", "bfloat16"), ("B", "float32")])
 def test_what_a_page_held_before_never_reaches_a_result(name, dtype, backend):

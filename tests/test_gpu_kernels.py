@@ -374,6 +374,69 @@ def test_long_portions_by_tiles(ops_for, monkeypatch, n_heads, n_kv, hd, page_si
         torch.testing.assert_close(got[r].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("first", [0, 30, 60, 90])
+def test_paged_attention_of_drawn_batches(ops_for, monkeypatch, first):
+    """Thirty batches a case with everything drawn at random: heads and groups, head sizes in steps of 16 up to 256,
+    the page, a window or none, and one to four requests (decoded tokens, short and long portions, from an empty
+    cache or deep in a request) or ten to twenty-four decoded tokens of uneven lengths; and, drawn too, whether
+    tiles' key ranges are cut however short, whether decoded rows beside tiles get planned splits, and whether short
+    portions beside deep rows still go to tiles. Rows at the starts, middles and ends of portions, at tile and page
+    edges and thirty drawn ones are compared with library attention over each row's own keys."""
+    from tiny_inference_server_amd.ops import hip_ops
+    ops = ops_for(torch.bfloat16)
+    for case in range(first, first + 30):
+        rng = random.Random(case)
+        n_kv, group = rng.choice([1, 1, 2, 3, 4]), rng.choice([1, 2, 3, 4, 4, 5, 8])
+        hd = rng.choice([16, 32, 48, 64, 80, 96, 128, 128, 160, 256])
+        page = rng.choice([16, 16, 32, 48, 64])
+        window = rng.choice([0, 0, 0, rng.randint(5, 900)])
+        n_heads = n_kv * group
+        n_req = rng.randint(1, 4) if rng.random() < 0.8 else rng.randint(10, 24)
+        segs = []
+        for i in range(n_req):
+            kind = rng.random()
+            if n_req > 4:
+                n, p0 = 1, (rng.randint(0, 1500) if rng.random() < 0.7 else rng.randint(0, 40))
+            elif kind < 0.3:
+                n, p0 = 1, rng.randint(0, 2500)
+            elif kind < 0.5:
+                n, p0 = rng.randint(2, 40), rng.randint(0, 1500)
+            elif kind < 0.8:
+                n, p0 = rng.randint(41, 700), rng.choice([0, 0, rng.randint(1, 1500)])
+            else:
+                n, p0 = rng.randint(700, 1500), rng.choice([0, rng.randint(1, 800)])
+            segs.append((i, p0, n))
+        with monkeypatch.context() as m:
+            if rng.random() < 0.4:
+                m.setattr(hip_ops, "_tiles_cut_pays", lambda *a: True)
+            if rng.random() < 0.5:
+                m.setattr(hip_ops, "_ATTN_PLANNED_BESIDE_FROM", 0.0)
+            if rng.random() < 0.5:
+                m.setattr(hip_ops, "_ATTN_TILE_MIN_WORK_MIXED", 0)
+            kv_lens = [p0 + n for _, p0, n in segs]
+            plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page, torch.bfloat16, seed=case * 7 + 1)
+            positions, row_seq, seq_rows = [], [], []
+            for s_, p0, n in segs:
+                seq_rows.append((len(positions), p0, n))
+                positions += list(range(p0, p0 + n)); row_seq += [s_] * n
+            R = len(positions)
+            q = rnd((R, n_heads * hd), torch.bfloat16, case * 7 + 2)
+            batch = SimpleNamespace(positions=torch.tensor(positions, dtype=torch.int32).cuda(),
+                                    row_seq=torch.tensor(row_seq, dtype=torch.int32).cuda(),
+                                    block_tables={"g": tables.cuda()}, max_kv_len=max(kv_lens), extras={},
+                                    n_rows=R, max_seq_rows=max(n for _, _, n in segs), seq_rows=seq_rows)
+            got = ops.paged_attention(q.cuda(), plane.cuda(), batch, "g", n_heads, n_kv, hd, window=window).cpu()
+        what = f"case {case}: heads {n_heads}/{n_kv} of {hd}, page {page}, window {window}, (first, rows) {[s[1:] for s in segs]}"
+        assert torch.isfinite(got.float()).all(), what
+        rows = set(rng.sample(range(R), min(R, 30)))
+        for start, p0, n in seq_rows:
+            rows |= {start, start + n - 1, start + n // 2} | {start + e for e in (15, 16, 31, 32, 63, 64, 127, 128) if e < n}
+        for r in sorted(rows):
+            want = dense_reference(q[r].view(n_heads, hd), ks[row_seq[r]], vs[row_seq[r]], group, positions[r], window)
+            torch.testing.assert_close(got[r].view(n_heads, hd).double(), want, rtol=2e-2, atol=2e-2,
+                                       msg=lambda m_: f"{what}, row {r} at position {positions[r]}: {m_}")
+
+
 @pytest.mark.parametrize("splits", [False, True])
 def test_a_tile_sees_a_far_key_and_a_rows_own_key(ops_for, monkeypatch, splits):
     """Two scores are made to stand out in a long portion: a key far back (in an early split of the tile's keys, when

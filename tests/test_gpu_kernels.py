@@ -836,6 +836,36 @@ def test_projection_with_rotary_and_cache_write(ops_for, dtype, M, n_heads, n_kv
         torch.testing.assert_close(got.double().view(M, n_heads, hd), q * c + rot * s, **t)
 
 
+@pytest.mark.parametrize("first", [0, 60, 120])
+def test_products_of_drawn_shapes(ops_for, first):
+    """Sixty products a case with the rows (1 to 2,100), both widths (aligned to 16, 8, 4 or 2, or to nothing) and the
+    kind (plain, with residual, with the norm in front, gated, 32-bit results) drawn at random: whichever kernel the
+    route picks for a shape (few rows, tiles, or the plain one for unaligned operands), the result is the reference's."""
+    ops, ref = ops_for(torch.bfloat16), TorchOps(dtype=torch.bfloat16)
+    for case in range(first, first + 60):
+        rng = random.Random(5000 + case)
+        M = rng.choice([rng.randint(1, 8), rng.randint(9, 32), rng.randint(33, 128), rng.randint(129, 600), rng.randint(600, 2100)])
+        N = rng.choice([rng.randint(1, 64) * 4, rng.randint(8, 300) * 8, rng.randint(100, 1100) * 8, rng.randint(1, 2000) * 2,
+                        rng.randint(1, 3000)])
+        K = rng.choice([rng.randint(1, 40) * 8, rng.randint(8, 560) * 8, rng.randint(8, 280) * 16, rng.randint(1, 500) * 2])
+        kind = rng.choice(["plain", "residual", "norm", "norm+residual", "f32", "gate", "norm+gate"])
+        if "gate" in kind:
+            N = max(2, N // 2 * 2)
+        x, w = rnd((M, K), torch.bfloat16, case * 3 + 1, 2.0), rnd((N, K), torch.bfloat16, case * 3 + 2, K ** -0.5)
+        gain, res = 1 + 0.1 * rnd((K,), torch.float32, case * 3 + 3), rnd((M, N), torch.bfloat16, case * 3 + 4)
+        rms_there, rms_here = ((gain.cuda(), 1e-5), (gain, 1e-5)) if "norm" in kind else (None, None)
+        if "gate" in kind:
+            got, want = ops.linear_swiglu(x.cuda(), w.cuda(), rms=rms_there), ref.linear_swiglu(x, w, rms=rms_here)
+        elif kind == "f32":
+            got, want = ops.linear(x.cuda(), w.cuda(), out_dtype=torch.float32), ref.linear(x, w, out_dtype=torch.float32)
+        else:
+            with_res = "residual" in kind
+            got = ops.linear(x.cuda(), w.cuda(), residual=res.clone().cuda() if with_res else None, rms=rms_there)
+            want = ref.linear(x, w, residual=res.clone() if with_res else None, rms=rms_here)
+        torch.testing.assert_close(got.cpu().float(), want.float(), rtol=3e-2, atol=3e-2,
+                                   msg=lambda m_: f"case {case}: {kind}, {M} rows, {N} out, {K} in: {m_}")
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 20, 40, 70])
 def test_skinny_product_with_two_column_tiles_a_workgroup(ops_for, M):
     """Very wide matrices give a workgroup of the staged kernel two column tiles. Forced here at a small width that

@@ -236,6 +236,43 @@ def test_drawn_configurations_under_drawn_schedules(seed, backend):
     assert eng.free_pages() == eng.total_pages()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(16))
+def test_drawn_configurations_decoding_together_through_captured_steps(seed):
+    """Drawn sizes again, now for the steps that serving is made of: one to twenty requests' prompts (half of the
+    time most of them short beside a few long ones, so that splits are planned request by request), then all of them
+    decoding together for up to thirty steps, which are captured and replayed (more than eight requests: the shapes
+    with filler lines); one request may end early, so that the step's shape changes under way. Every page starts out
+    full of NaN. The first stage's logits against the plain implementation."""
+    import random
+    name = f"together{seed}"
+    rng, H.TINY[name] = drawn_configuration(seed + 500)
+    cfg = H.TINY[name]["cfg"]
+    dtype = rng.choice(["bfloat16", "bfloat16", "float32"])
+    n_req, n_dec, uneven = rng.choice([1, 2, 3, 5, 8, 9, 12, 17, 20]), rng.randint(8, 30), rng.random() < 0.5
+    lens = [rng.randint(cfg.mtp_heads + 3, 20 if (uneven and i % 3) else min(150, cfg.max_context - n_dec - 4))
+            for i in range(n_req)]
+    reqs = {f"r{i}": H.random_ids(cfg.vocab_size, n + n_dec, seed * 100 + i) for i, n in enumerate(lens)}
+    steps = [{"step": i, "entries": [{"id": rid, "tokens": ids[:lens[i]], "want": [lens[i] - 1]}], "end": []}
+             for i, (rid, ids) in enumerate(reqs.items())]
+    leave = rng.choice([None, rng.randint(2, n_dec - 2)]) if n_req > 2 else None      # the step after which r1 is gone
+    for k in range(n_dec):
+        live = [(i, rid) for i, rid in enumerate(reqs) if not (leave is not None and i == 1 and k >= leave)]
+        ended = (["r1"] if leave is not None and k == leave - 1 else []) + ([rid for _, rid in live] if k == n_dec - 1 else [])
+        steps.append({"step": len(steps), "end": ended,
+                      "entries": [{"id": rid, "tokens": [reqs[rid][lens[i] + k]], "want": [0]} for i, rid in live]})
+    if leave is not None:
+        reqs["r1"] = reqs["r1"][:lens[1] + leave]
+    folder, eng = make_engine(name, dtype, "hip", max_tokens=sum(-(-len(v) // 64) * 64 for v in reqs.values()),
+                              max_requests=max(4, n_req))
+    H.fill_cache_with_nan(eng)
+    main, _ = H.run_trace(eng, steps, heads=False)
+    assert eng.graph_replays >= n_dec // 2
+    H.compare_with_plain(folder, reqs, main, {}, TOL[dtype] * scale_of(folder, reqs), 0)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages()
+
+
 @pytest.mark.parametrize("backend", backends())
 @pytest.mark.parametrize("name,dtype", [("D", "bfloat16"), ("B", "float32")])
 def test_what_a_page_held_before_never_reaches_a_result(name, dtype, backend):

@@ -109,6 +109,56 @@ def test_scheduler_at_the_headline_geometry_with_fourteen_sampled_requests_on_a_
     assert eng.free_pages() == eng.total_pages() and eng.cache.n_live == 0
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_scheduler_on_drawn_configurations_with_drawn_sampling(seed):
+    """Every size of the model drawn at random, then the scheduler's own knobs (requests, slots, token budget, plan,
+    a pool from too small for all to ample, heads run or not) and each request's sampling (arg-max, temperatures,
+    top-k, top-p, repetition penalty) drawn too, in 32-bit on a pool full of NaN: every sampled token is the plain
+    rule's draw on the plain model's logits (server.py:22-50) up to rounding at a boundary of the cumulative
+    distribution, every arg-max token the plain arg-max where that is clear, and nothing is left in the cache."""
+    import random
+    from test_engine_schedules import drawn_configuration
+    from tiny_inference_server_amd.engine import Engine
+    from tiny_inference_server_amd.engine.scheduler import Request, Scheduler
+    name = f"scheduled{seed}"
+    rng, H.TINY[name] = drawn_configuration(seed + 900)
+    cfg, page = H.TINY[name]["cfg"], H.TINY[name]["page_size"]
+    n_req = rng.choice([2, 4, 6, 10, 14])
+    prompts = [H.random_ids(cfg.vocab_size, rng.randint(1, 60), seed * 50 + i) for i in range(n_req)]
+    params = [SamplingParams(max_new_tokens=rng.randint(3, 20), temperature=rng.choice([0.0, 0.3, 0.8, 1.0]),
+                             top_k=rng.choice([0, 0, 5, 40]), top_p=rng.choice([1.0, 1.0, 0.9, 0.5]),
+                             rep_penalty=rng.choice([1.0, 1.3]), seed=seed * 10 + i, ignore_eos=True) for i in range(n_req)]
+    sizes = [len(p) + sp.max_new_tokens for p, sp in zip(prompts, params)]
+    pool = max(-(-max(sizes) // page) * page + page, int(sum(sizes) * rng.choice([0.4, 0.7, 1.2])) // page * page)
+    plan, heads, max_batch = rng.choice(["cur", "final"]), rng.random() < 0.5, rng.choice([2, 4, n_req])
+    budget = max(rng.choice([8, 24, 64, 256]), max_batch)
+    folder = H.model_folder(name, "float32")
+    eng = Engine(folder, dtype="float32", page_size=page, max_tokens=pool, max_requests=max_batch, run_heads=heads)
+    H.fill_cache_with_nan(eng)
+    s = Scheduler(eng, max_batch=max_batch, token_budget=budget, plan=plan)
+    reqs = [Request(p, sp) for p, sp in zip(prompts, params)]
+    for r in reqs:
+        s.submit(r)
+    s.run()
+    sampled = [i for i, sp in enumerate(params) if sp.temperature > 0.0]
+    H.check_sampled_tokens(folder, [prompts[i] for i in sampled], [params[i] for i in sampled],
+                           [reqs[i].out_ids() for i in sampled], slack=1e-4)
+    model_cfg, w = pm.read_model_folder(folder)
+    for i, sp in enumerate(params):
+        out = reqs[i].out_ids()
+        assert len(out) == sp.max_new_tokens
+        if sp.temperature > 0.0 or sp.rep_penalty != 1.0:
+            continue
+        ids = list(prompts[i])
+        for t in out:
+            lg = pm.logits_of(pm.trunk_hidden(ids, w, model_cfg)[-1:], w, model_cfg)[0]
+            top2 = torch.topk(lg, 2).values
+            assert t == int(lg.argmax()) or (top2[0] - top2[1]).item() < 1e-3
+            ids.append(t)
+    eng.cache.check()
+    assert eng.free_pages() == eng.total_pages() and eng.cache.n_live == 0
+
+
 def test_temperature_sampling_with_seeded_streams():
     """Tiny B's workload: temperature 0.8, seed 0, mixed chunked prefill and decode; token by token the draw is the
     plain rule's (server.py:22-50) on the plain logits with the request's own uniform number."""
